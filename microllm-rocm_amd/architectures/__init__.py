@@ -1,2 +1,2 @@
 """Architectures this package provides; importing the package registers them."""
-from . import gupitar, qwen2, siditar  # noqa: F401
+from . import gupitar, qwen2, siditar, zabozen  # noqa: F401

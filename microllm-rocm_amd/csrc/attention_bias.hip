@@ -65,7 +65,8 @@ bias_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
                       const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ seq_of_token,
                       const int32_t* __restrict__ positions, const float* __restrict__ bias, int longest,
                       const float* __restrict__ sink, T* __restrict__ out, int64_t out_stride, int heads, int kv_heads,
-                      int key_dim, int value_dim, int page_size, float scale, float out_scale) {
+                      int key_dim, int value_dim, int page_size, float scale, float out_scale,
+                      const float* __restrict__ slopes, int window) {
     extern __shared__ float q_row[];
     const int token = blockIdx.x / heads;
     const int head = blockIdx.x % heads;
@@ -83,26 +84,30 @@ bias_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
     float acc[kMaxValueChannelsALane] = {0.0f, 0.0f, 0.0f, 0.0f};
     const int64_t key_row = static_cast<int64_t>(kv_heads) * key_dim;
     const int64_t value_row = static_cast<int64_t>(kv_heads) * value_dim;
-    for (int first = 0; first <= position; first += kBiasKeyTile) {
+    const float slope = slopes ? slopes[head] : 0.0f;
+    const int low = window > 0 ? max(0, position - window + 1) : 0;     // the oldest key seen
+    for (int first = low / kBiasKeyTile * kBiasKeyTile; first <= position; first += kBiasKeyTile) {
         const int j = first + lane;
         float score = -INFINITY;
         int64_t place = 0;
-        if (j <= position) {
+        const bool seen = j >= low && j <= position;
+        if (seen) {
             place = static_cast<int64_t>(table[j / page_size]) * page_size + j % page_size;
             const T* key = k_pages + place * key_row + static_cast<int64_t>(kv_head) * key_dim;
             score = dot_row<T>(key, q_row, key_dim) * scale;
             if (bias) score += bias[static_cast<int64_t>(min(position - j, longest)) * heads + head];
+            if (slopes) score -= slope * static_cast<float>(position - j);
         }
         const float tile_max = wave_max(score);
         const float new_max = fmaxf(running_max, tile_max);
         const float keep = running_max == -INFINITY ? 0.0f : expf(running_max - new_max);
-        const float weight = j <= position ? expf(score - new_max) : 0.0f;
+        const float weight = seen ? expf(score - new_max) : 0.0f;
         running_sum = running_sum * keep + wave_sum(weight);
         running_max = new_max;
 #pragma unroll
         for (int m = 0; m < kMaxValueChannelsALane; ++m) acc[m] *= keep;
         const int in_tile = min(kBiasKeyTile, position - first + 1);
-        for (int n = 0; n < in_tile; ++n) {
+        for (int n = max(0, low - first); n < in_tile; ++n) {
             const float w = __shfl(weight, n, kWave);
             const int64_t at = __shfl(place, n, kWave);
             const T* value = v_pages + at * value_row + static_cast<int64_t>(kv_head) * value_dim;
@@ -130,28 +135,30 @@ qk_norm_store_kernel(const float* __restrict__ qkv, int n_parts, int64_t part_st
                      const float* __restrict__ k_weight, float eps, const int32_t* __restrict__ positions,
                      const int32_t* __restrict__ slot_mapping, float temp_coef, int temp_every, T* __restrict__ q_out,
                      T* __restrict__ k_pages, T* __restrict__ v_pages, int heads, int kv_heads, int key_dim, int value_dim,
-                     int tiled_page_size) {
-    const int vectors = heads + 2 * kv_heads;
+                     int tiled_page_size, const float* __restrict__ bias, int normed, int queries_only) {
+    const int vectors = queries_only ? heads : heads + 2 * kv_heads;
     const int token = blockIdx.x / vectors;
     const int which = blockIdx.x % vectors;
     const int lane = threadIdx.x;
-    const int row_width = (heads + kv_heads) * key_dim + kv_heads * value_dim;
+    const int row_width = queries_only ? heads * key_dim : (heads + kv_heads) * key_dim + kv_heads * value_dim;
     const float* row = qkv + static_cast<int64_t>(token) * row_width;
     const bool is_q = which < heads, is_k = !is_q && which < heads + kv_heads;
     const int head = is_q ? which : (is_k ? which - heads : which - heads - kv_heads);
     const int dim = (is_q || is_k) ? key_dim : value_dim;
     const int offset = is_q ? head * key_dim : (is_k ? (heads + head) * key_dim : (heads + kv_heads) * key_dim + head * value_dim);
-    const int slot = slot_mapping[token];
+    const int slot = is_q ? 0 : slot_mapping[token];
     if (!is_q && slot < 0) return;
     float squares = 0.0f;
     for (int c = lane; c < dim; c += kWave) {
         float value = row[offset + c];
         for (int part = 1; part < n_parts; ++part) value += row[part * part_stride + offset + c];
+        if (bias) value += bias[offset + c];
         squares += value * value;
     }
     const float* weight = is_q ? q_weight : (is_k ? k_weight : nullptr);
+    const bool norm = normed && (is_q || is_k);
     float factor = 1.0f;
-    if (weight != nullptr) factor = 1.0f / sqrtf(wave_sum(squares) / static_cast<float>(dim) + eps);
+    if (norm) factor = 1.0f / sqrtf(wave_sum(squares) / static_cast<float>(dim) + eps);
     if (is_q && temp_coef != 0.0f) {
         const int steps = (positions[token] + 1) / temp_every;
         factor *= 1.0f + temp_coef * static_cast<float>(log(static_cast<double>(steps) + 1.0));
@@ -167,7 +174,8 @@ qk_norm_store_kernel(const float* __restrict__ qkv, int n_parts, int64_t part_st
     for (int c = lane; c < dim; c += kWave) {
         float value = row[offset + c];
         for (int part = 1; part < n_parts; ++part) value += row[part * part_stride + offset + c];
-        const T rounded = from_float<T>(weight ? value * factor * weight[c] : value);
+        if (bias) value += bias[offset + c];
+        const T rounded = from_float<T>(norm ? (weight ? value * factor * weight[c] : value * factor) : value);
         if (tiled) {
             if (is_k) k_pages[layout.k_at(page, head, in_page, c)] = rounded;
             else v_pages[layout.v_at(page, head, in_page, c)] = rounded;
@@ -186,27 +194,29 @@ extern "C" {
 int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const float* q_weight, const float* k_weight,
                       float eps, const int32_t* positions, const int32_t* slot_mapping, float temp_coef, int temp_every,
                       void* q_out, void* k_pages, void* v_pages, int dtype, int n_tokens, int heads, int kv_heads, int key_dim,
-                      int value_dim, int tiled_page_size, hipStream_t stream) {
+                      int value_dim, int tiled_page_size, const float* bias, int normed, int queries_only, hipStream_t stream) {
     MLL_REQUIRE(tiled_page_size == 0 || (tiled_page_size > 0 && tiled_page_size % 16 == 0 && key_dim == value_dim),
                 "qk_norm_store: tiled pages hold a multiple of 16 positions and keys and values of one width");
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0, "qk_norm_store: sizes must be positive");
     MLL_REQUIRE(n_parts >= 1, "qk_norm_store: at least one part");
     MLL_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qk_norm_store: norm weights for queries and keys, or for neither");
-    MLL_REQUIRE(q_weight == nullptr || eps > 0.0f, "qk_norm_store: eps must be positive");
+    MLL_REQUIRE(!normed || eps > 0.0f, "qk_norm_store: eps must be positive");
+    MLL_REQUIRE(normed || q_weight == nullptr, "qk_norm_store: norm weights without a norm");
+    MLL_REQUIRE(queries_only || (slot_mapping != nullptr && k_pages != nullptr && v_pages != nullptr), "qk_norm_store: keys and values need pages and slots");
     MLL_REQUIRE(temp_coef == 0.0f || temp_every > 0, "qk_norm_store: the factor by position needs a positive step");
     if (n_tokens == 0) return 0;
-    const int64_t blocks = static_cast<int64_t>(n_tokens) * (heads + 2 * kv_heads);
+    const int64_t blocks = static_cast<int64_t>(n_tokens) * (queries_only ? heads : heads + 2 * kv_heads);
     MLL_REQUIRE(blocks < (1ll << 31), "qk_norm_store: too many rows for one launch");
     if (dtype == kF32) {
         qk_norm_store_kernel<float><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
             qkv, n_parts, part_stride, q_weight, k_weight, eps, positions, slot_mapping, temp_coef, temp_every,
             static_cast<float*>(q_out), static_cast<float*>(k_pages), static_cast<float*>(v_pages), heads, kv_heads, key_dim, value_dim,
-            tiled_page_size);
+            tiled_page_size, bias, normed, queries_only);
     } else if (dtype == kBF16) {
         qk_norm_store_kernel<bf16><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
             qkv, n_parts, part_stride, q_weight, k_weight, eps, positions, slot_mapping, temp_coef, temp_every,
             static_cast<bf16*>(q_out), static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), heads, kv_heads, key_dim, value_dim,
-            tiled_page_size);
+            tiled_page_size, bias, normed, queries_only);
     } else {
         return fail("qk_norm_store: unknown dtype");
     }
@@ -216,7 +226,8 @@ int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const 
 int mll_bias_attention(const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_width,
                        const int32_t* seq_of_token, const int32_t* positions, const float* bias, int longest,
                        const float* sink, void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int kv_heads,
-                       int key_dim, int value_dim, int page_size, float scale, float out_scale, hipStream_t stream) {
+                       int key_dim, int value_dim, int page_size, float scale, float out_scale, const float* slopes, int window,
+                       hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0 && page_size > 0 && table_width > 0,
                 "bias_attention: sizes must be positive");
     MLL_REQUIRE(heads % kv_heads == 0, "bias_attention: heads must divide into kv heads");
@@ -232,12 +243,12 @@ int mll_bias_attention(const void* q, const void* k_pages, const void* v_pages, 
         bias_attention_kernel<float><<<static_cast<unsigned>(blocks), kWave, lds, stream>>>(
             static_cast<const float*>(q), static_cast<const float*>(k_pages), static_cast<const float*>(v_pages), block_table,
             table_width, seq_of_token, positions, bias, longest, sink, static_cast<float*>(out), out_stride, heads, kv_heads,
-            key_dim, value_dim, page_size, scale, out_scale);
+            key_dim, value_dim, page_size, scale, out_scale, slopes, window);
     } else if (dtype == kBF16) {
         bias_attention_kernel<bf16><<<static_cast<unsigned>(blocks), kWave, lds, stream>>>(
             static_cast<const bf16*>(q), static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages), block_table,
             table_width, seq_of_token, positions, bias, longest, sink, static_cast<bf16*>(out), out_stride, heads, kv_heads,
-            key_dim, value_dim, page_size, scale, out_scale);
+            key_dim, value_dim, page_size, scale, out_scale, slopes, window);
     } else {
         return fail("bias_attention: unknown dtype");
     }

@@ -173,6 +173,16 @@ __global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__
     if (index < count) h[index] += to_float(delta[index]);
 }
 
+__global__ void add_bias_kernel(float* __restrict__ values, const float* __restrict__ bias, int64_t count, int width) {
+    const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index < count) values[index] += bias[index % width];
+}
+
+__global__ void softcap_kernel(float* __restrict__ values, int64_t count, float cap) {
+    const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index < count) values[index] = cap * tanhf(values[index] / cap);
+}
+
 // ---------------------------------------------------------------------------------------------
 // cos and sin of position * inv_freq for every token of a step: angles in float64, so that the float32 values
 // are the correctly rounded ones for any position. out[token][pair] = (cos, sin).
@@ -463,6 +473,25 @@ int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int wid
         return fail("residual_add: unknown dtype");
     }
     return check_launch("residual_add");
+}
+
+int mll_add_bias(float* values, const float* bias, int64_t n_rows, int width, hipStream_t stream) {
+    MLL_REQUIRE(width > 0 && n_rows >= 0, "add_bias: sizes must be positive");
+    const int64_t count = n_rows * width;
+    if (count == 0) return 0;
+    const int64_t blocks = (count + 255) / 256;
+    MLL_REQUIRE(blocks < (1ll << 31), "add_bias: too many values for one launch");
+    add_bias_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(values, bias, count, width);
+    return check_launch("add_bias");
+}
+
+int mll_softcap(float* values, int64_t count, float cap, hipStream_t stream) {
+    MLL_REQUIRE(cap > 0.0f, "softcap: the cap must be positive");
+    if (count <= 0) return 0;
+    const int64_t blocks = (count + 255) / 256;
+    MLL_REQUIRE(blocks < (1ll << 31), "softcap: too many values for one launch");
+    softcap_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(values, count, cap);
+    return check_launch("softcap");
 }
 
 int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t partial_stride, int dtype,

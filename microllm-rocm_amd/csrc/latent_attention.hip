@@ -31,6 +31,7 @@ latent_prepare_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     const int thread = threadIdx.x;
     const float* row = proj + static_cast<int64_t>(token) * proj_stride;
     if (which == 0) {
+        if (q_rank <= 0) return;        // the queries have no latent of their own
         float squares = 0.0f;
         for (int c = thread; c < q_rank; c += kPrepareThreads) squares = fmaf(row[q_at + c], row[q_at + c], squares);
         const float factor = 1.0f / sqrtf(block_sum(squares, scratch) / static_cast<float>(q_rank) + eps);
@@ -74,12 +75,12 @@ latent_prepare_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
 // the unrotated part as [head][token][dim] for such a product.
 template <typename T>
 __global__ void __launch_bounds__(kWave)
-latent_query_kernel(const float* __restrict__ q, int n_tokens, int heads, int dim, int rot_dim, int kv_rank,
+latent_query_kernel(const float* __restrict__ q, int64_t q_stride, int n_tokens, int heads, int dim, int rot_dim, int kv_rank,
                     const float* __restrict__ cos_sin, const T* __restrict__ folded, T* __restrict__ flat_out,
                     T* __restrict__ q_full) {
     const int token = blockIdx.x / heads, head = blockIdx.x % heads;
     const int lane = threadIdx.x;
-    const float* row = q + (static_cast<int64_t>(token) * heads + head) * (dim + rot_dim);
+    const float* row = q + static_cast<int64_t>(token) * q_stride + static_cast<int64_t>(head) * (dim + rot_dim);
     T* to = q_full + (static_cast<int64_t>(token) * heads + head) * (kv_rank + rot_dim);
     const int half = rot_dim / 2;
     for (int i = lane; i < half; i += kWave) {
@@ -114,7 +115,7 @@ template <typename X, typename W, typename O, int SLICES>
 __global__ void __launch_bounds__(SLICES * kWave)
 head_product_kernel(const X* __restrict__ x, int64_t x_token_stride, int64_t x_head_stride, const W* __restrict__ w,
                     O* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride, const float* __restrict__ gate,
-                    int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out) {
+                    int64_t gate_stride, int gate_a_head, int n_tokens, int heads, int n_in, int n_out) {
     extern __shared__ float x_rows[];      // [kHeadProductRows][tile], then [slices - 1][kHeadProductRows][64] partial sums
     constexpr int kOwn = kHeadProductSlices / SLICES;       // quarters a thread walks
     constexpr int kAhead = 16;                              // weight loads a thread of the four-wave kernel has on their way
@@ -183,7 +184,7 @@ head_product_kernel(const X* __restrict__ x, int64_t x_token_stride, int64_t x_h
         for (int other = 1; other < kHeadProductSlices; ++other)
             value += SLICES == 1 ? acc[other % kOwn][r] : partial[((other - 1) * kHeadProductRows + r) * kWave + lane];
         if (gate != nullptr) {
-            const float g = gate[static_cast<int64_t>(first + r) * gate_stride + static_cast<int64_t>(head) * n_out + o];
+            const float g = gate[static_cast<int64_t>(first + r) * gate_stride + (gate_a_head ? head : static_cast<int64_t>(head) * n_out + o)];
             value *= 1.0f / (1.0f + expf(-g));
         }
         out[static_cast<int64_t>(first + r) * out_token_stride + static_cast<int64_t>(head) * out_head_stride + o] = from_float<O>(value);
@@ -193,13 +194,13 @@ head_product_kernel(const X* __restrict__ x, int64_t x_token_stride, int64_t x_h
 // out[t][h * n + c] = in[h][t][c] * sigmoid(gate[t][h * n + c]): the heads of a batched product side by side, gated.
 template <typename T>
 __global__ void __launch_bounds__(256)
-gate_heads_kernel(const T* __restrict__ in, const float* __restrict__ gate, int64_t gate_stride, T* __restrict__ out,
-                  int n_tokens, int heads, int n) {
+gate_heads_kernel(const T* __restrict__ in, const float* __restrict__ gate, int64_t gate_stride, int gate_a_head,
+                  T* __restrict__ out, int n_tokens, int heads, int n) {
     const int token = blockIdx.x;
     for (int column = threadIdx.x; column < heads * n; column += blockDim.x) {
         const int head = column / n, c = column % n;
         float value = to_float(in[(static_cast<int64_t>(head) * n_tokens + token) * n + c]);
-        if (gate != nullptr) value *= 1.0f / (1.0f + expf(-gate[static_cast<int64_t>(token) * gate_stride + column]));
+        if (gate != nullptr) value *= 1.0f / (1.0f + expf(-gate[static_cast<int64_t>(token) * gate_stride + (gate_a_head ? head : column)]));
         out[static_cast<int64_t>(token) * heads * n + column] = from_float<T>(value);
     }
 }
@@ -312,19 +313,19 @@ constexpr int kHeadProductFewRows = 64;     // up to this many tokens a step, fo
 
 template <typename X, typename W, typename O>
 int launch_head_product(const void* x, int64_t x_token_stride, int64_t x_head_stride, const void* w, void* out,
-                        int64_t out_token_stride, int64_t out_head_stride, const float* gate, int64_t gate_stride, int n_tokens,
-                        int heads, int n_in, int n_out, hipStream_t stream) {
+                        int64_t out_token_stride, int64_t out_head_stride, const float* gate, int64_t gate_stride, int gate_a_head,
+                        int n_tokens, int heads, int n_in, int n_out, hipStream_t stream) {
     const dim3 grid((n_out + kWave - 1) / kWave, heads, (n_tokens + kHeadProductRows - 1) / kHeadProductRows);
     const size_t staged = static_cast<size_t>(kHeadProductRows) * (n_in < kHeadProductTile ? n_in : kHeadProductTile);
     if (n_tokens <= kHeadProductFewRows) {
         const size_t lds = (staged + (kHeadProductSlices - 1) * kHeadProductRows * kWave) * sizeof(float);
         head_product_kernel<X, W, O, kHeadProductSlices><<<grid, kHeadProductSlices * kWave, lds, stream>>>(
             static_cast<const X*>(x), x_token_stride, x_head_stride, static_cast<const W*>(w), static_cast<O*>(out),
-            out_token_stride, out_head_stride, gate, gate_stride, n_tokens, heads, n_in, n_out);
+            out_token_stride, out_head_stride, gate, gate_stride, gate_a_head, n_tokens, heads, n_in, n_out);
     } else {
         head_product_kernel<X, W, O, 1><<<grid, kWave, staged * sizeof(float), stream>>>(
             static_cast<const X*>(x), x_token_stride, x_head_stride, static_cast<const W*>(w), static_cast<O*>(out),
-            out_token_stride, out_head_stride, gate, gate_stride, n_tokens, heads, n_in, n_out);
+            out_token_stride, out_head_stride, gate, gate_stride, gate_a_head, n_tokens, heads, n_in, n_out);
     }
     return check_launch("head_product");
 }
@@ -339,8 +340,8 @@ int mll_latent_prepare(const float* proj, int64_t proj_stride, int q_at, int q_r
                        int kv_rank, int rot_dim, const float* kv_weight, float eps, const float* cos_sin,
                        const int32_t* slot_mapping, void* q_latent, void* pages, void* k_pages, void* v_pages,
                        int tiled_page_size, int dtype, int n_tokens, hipStream_t stream) {
-    MLL_REQUIRE(n_tokens >= 0 && q_rank > 0 && q_weight != nullptr && q_latent != nullptr && eps > 0.0f,
-                "latent_prepare: the queries' latent needs a size, a weight and a place");
+    MLL_REQUIRE(n_tokens >= 0 && eps > 0.0f && (q_rank == 0 || (q_rank > 0 && q_weight != nullptr && q_latent != nullptr)),
+                "latent_prepare: the queries' latent needs a size, a weight and a place (size 0: there is none)");
     if (slot_mapping != nullptr) {
         MLL_REQUIRE(kv_rank > 0 && rot_dim > 0 && rot_dim % 2 == 0 && kv_weight != nullptr && cos_sin != nullptr,
                     "latent_prepare: the keys' latent needs its sizes (an even rotated part), a weight and cos/sin");
@@ -364,20 +365,21 @@ int mll_latent_prepare(const float* proj, int64_t proj_stride, int q_at, int q_r
     return check_launch("latent_prepare");
 }
 
-int mll_latent_query(const float* q, int n_tokens, int heads, int dim, int rot_dim, int kv_rank, const float* cos_sin,
+int mll_latent_query(const float* q, int64_t q_stride, int n_tokens, int heads, int dim, int rot_dim, int kv_rank, const float* cos_sin,
                      const void* folded, void* flat_out, void* q_full, int dtype, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && dim > 0 && rot_dim > 0 && rot_dim % 2 == 0 && kv_rank > 0 && cos_sin != nullptr,
                 "latent_query: sizes must be positive, the rotated part even");
+    MLL_REQUIRE(q_stride >= static_cast<int64_t>(heads) * (dim + rot_dim), "latent_query: the queries' rows overlap");
     if (n_tokens == 0) return 0;
     const int64_t blocks = static_cast<int64_t>(n_tokens) * heads;
     MLL_REQUIRE(blocks < (1ll << 31), "latent_query: too many rows for one launch");
     if (dtype == kF32) {
         latent_query_kernel<float><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
-            q, n_tokens, heads, dim, rot_dim, kv_rank, cos_sin, static_cast<const float*>(folded), static_cast<float*>(flat_out),
+            q, q_stride, n_tokens, heads, dim, rot_dim, kv_rank, cos_sin, static_cast<const float*>(folded), static_cast<float*>(flat_out),
             static_cast<float*>(q_full));
     } else if (dtype == kBF16) {
         latent_query_kernel<bf16><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
-            q, n_tokens, heads, dim, rot_dim, kv_rank, cos_sin, static_cast<const bf16*>(folded), static_cast<bf16*>(flat_out),
+            q, q_stride, n_tokens, heads, dim, rot_dim, kv_rank, cos_sin, static_cast<const bf16*>(folded), static_cast<bf16*>(flat_out),
             static_cast<bf16*>(q_full));
     } else {
         return fail("latent_query: unknown dtype");
@@ -387,13 +389,13 @@ int mll_latent_query(const float* q, int n_tokens, int heads, int dim, int rot_d
 
 int mll_head_product(const void* x, int x_dtype, int64_t x_token_stride, int64_t x_head_stride, const void* w, int w_dtype,
                      void* out, int out_dtype, int64_t out_token_stride, int64_t out_head_stride, const float* gate,
-                     int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream) {
+                     int64_t gate_stride, int gate_a_head, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && n_in > 0 && n_out > 0, "head_product: sizes must be positive");
     MLL_REQUIRE(heads < 65536 && (n_tokens + kHeadProductRows - 1) / kHeadProductRows < 65536, "head_product: too many heads or rows for one launch");
     if (n_tokens == 0) return 0;
 #define MLL_HEAD_PRODUCT(X, W, O)                                                                                          \
     return launch_head_product<X, W, O>(x, x_token_stride, x_head_stride, w, out, out_token_stride, out_head_stride, gate, \
-                                        gate_stride, n_tokens, heads, n_in, n_out, stream)
+                                        gate_stride, gate_a_head, n_tokens, heads, n_in, n_out, stream)
     if (x_dtype == kF32 && w_dtype == kF32 && out_dtype == kF32) MLL_HEAD_PRODUCT(float, float, float);
     if (x_dtype == kF32 && w_dtype == kBF16 && out_dtype == kBF16) MLL_HEAD_PRODUCT(float, bf16, bf16);
     if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kBF16) MLL_HEAD_PRODUCT(bf16, bf16, bf16);
@@ -428,14 +430,14 @@ int mll_latent_attention(const void* q_full, const void* pages, const int32_t* b
     return check_launch("latent_attention");
 }
 
-int mll_gate_heads(const void* in, const float* gate, int64_t gate_stride, void* out, int dtype, int n_tokens, int heads, int n,
-                   hipStream_t stream) {
+int mll_gate_heads(const void* in, const float* gate, int64_t gate_stride, int gate_a_head, void* out, int dtype, int n_tokens,
+                   int heads, int n, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && n > 0, "gate_heads: sizes must be positive");
     if (n_tokens == 0) return 0;
     if (dtype == kF32) {
-        gate_heads_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(in), gate, gate_stride, static_cast<float*>(out), n_tokens, heads, n);
+        gate_heads_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(in), gate, gate_stride, gate_a_head, static_cast<float*>(out), n_tokens, heads, n);
     } else if (dtype == kBF16) {
-        gate_heads_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(in), gate, gate_stride, static_cast<bf16*>(out), n_tokens, heads, n);
+        gate_heads_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(in), gate, gate_stride, gate_a_head, static_cast<bf16*>(out), n_tokens, heads, n);
     } else {
         return fail("gate_heads: unknown dtype");
     }

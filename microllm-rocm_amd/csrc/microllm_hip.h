@@ -26,6 +26,19 @@ int mll_rms_norm(float* h, const void* delta, int delta_dtype, int n_partials, i
                  const int32_t* rows, const float* weight, float eps,
                  void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream);
 
+// d = the delta's parts added in order; v = h[r] + mult * d * rsqrt(mean(d^2) + after_eps) * after_weight; if write_h,
+// h[r] = v; out[i] = v * rsqrt(mean(v^2) + eps) * weight (weight null: no output). A sublayer's result that is normed
+// itself before it joins the stream, fused with the norm that follows (csrc/norm_after.hip).
+int mll_rms_norm_after(float* h, const void* delta, int delta_dtype, int n_partials, int64_t partial_stride,
+                       const int32_t* rows, const float* after_weight, float after_eps, float mult, const float* weight,
+                       float eps, void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream);
+
+// values[r][c] += bias[c] for n_rows rows of `width` float32 values, in place.
+int mll_add_bias(float* values, const float* bias, int64_t n_rows, int width, hipStream_t stream);
+
+// values[i] = cap * tanh(values[i] / cap), in place, float32.
+int mll_softcap(float* values, int64_t count, float cap, hipStream_t stream);
+
 // Adds a pending delta into the residual stream: h[r] += delta[r] for all rows.
 int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int width, hipStream_t stream);
 
@@ -269,7 +282,9 @@ int mll_clamped_glu(const float* gate_up, void* out, int dtype, int n_tokens, in
 
 // qkv[t] = [q (heads * key_dim) | k (kv_heads * key_dim) | v (kv_heads * value_dim)] in float32, perhaps in
 // n_parts parts that are added in order. Queries and keys are divided by their root mean square over their head
-// (+ eps inside the root) and multiplied by q_weight / k_weight [key_dim] (both null: no norm); queries are then
+// (+ eps inside the root) if `normed`, and multiplied by q_weight / k_weight [key_dim] (both null: no weight); `bias`
+// (nullable, one number a column of a row) is added first; with queries_only a row holds queries alone and nothing
+// is stored; queries are then
 // multiplied by 1 + temp_coef * ln((p + 1) / temp_every + 1) (whole-number division) at position p
 // (temp_coef 0: not). Queries go to q_out [t][heads][key_dim]; keys and values into the pages
 // [slot][kv_head][dim] at slot_mapping[t] (negative: not stored), or, with tiled_page_size > 0 (the positions of a
@@ -277,16 +292,18 @@ int mll_clamped_glu(const float* gate_up, void* out, int dtype, int n_tokens, in
 int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const float* q_weight, const float* k_weight,
                       float eps, const int32_t* positions, const int32_t* slot_mapping, float temp_coef, int temp_every,
                       void* q_out, void* k_pages, void* v_pages, int dtype, int n_tokens, int heads, int kv_heads, int key_dim,
-                      int value_dim, int tiled_page_size, hipStream_t stream);
+                      int value_dim, int tiled_page_size, const float* bias, int normed, int queries_only, hipStream_t stream);
 
 // Causal attention of every token over its request's pages: score_j = (q . k_j) * scale + bias[min(p - j, longest)][head]
-// (bias null: none; float32 [longest + 1][heads]); softmax over j <= p with exp(sink[head]) added to the denominator
+// (bias null: none; float32 [longest + 1][heads]) - slopes[head] * (p - j) (slopes null: none); softmax over j <= p
+// (with window > 0: p - window < j <= p) with exp(sink[head]) added to the denominator
 // (sink null: not); out[t][head] = out_scale * sum_j weight_j v_j, rows out_stride elements apart.
 // A token whose seq_of_token is negative is skipped. The order of every sum depends on p alone.
 int mll_bias_attention(const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_width,
                        const int32_t* seq_of_token, const int32_t* positions, const float* bias, int longest,
                        const float* sink, void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int kv_heads,
-                       int key_dim, int value_dim, int page_size, float scale, float out_scale, hipStream_t stream);
+                       int key_dim, int value_dim, int page_size, float scale, float out_scale, const float* slopes, int window,
+                       hipStream_t stream);
 
 // ---- gated linear attention --------------------------------------------------------------------------------
 
@@ -312,7 +329,7 @@ int mll_gla_gate(const float* o, const float* proj, int64_t proj_stride, int gat
 
 // ---- attention through latents (csrc/latent_attention.hip) ----------------------------------------------------
 
-// proj[t] holds, in float32, the queries' down projection at q_at (q_rank wide) and the keys' and values' at kv_at
+// proj[t] holds, in float32, the queries' down projection at q_at (q_rank wide; 0: the queries have no latent) and the keys' and values' at kv_at
 // (kv_rank, then rot_dim). q_latent[t] = proj / rms * q_weight in `dtype`. With slot_mapping (null: the layer stores
 // nothing): the first kv_rank entries / rms * kv_weight and the last rot_dim turned by the split-half rule with
 // cos_sin [t][rot_dim / 2][2] go to slot slot_mapping[t] (negative: not stored) of `pages` [slot][kv_rank + rot_dim],
@@ -323,22 +340,23 @@ int mll_latent_prepare(const float* proj, int64_t proj_stride, int q_at, int q_r
                        const int32_t* slot_mapping, void* q_latent, void* pages, void* k_pages, void* v_pages,
                        int tiled_page_size, int dtype, int n_tokens, hipStream_t stream);
 
-// q: float32 [t][head][dim | rot_dim]. q_full [t][head][kv_rank | rot_dim] in `dtype` gets the rotated part turned;
+// q: float32 [t][head][dim | rot_dim], rows q_stride elements apart. q_full [t][head][kv_rank | rot_dim] in `dtype` gets the rotated part turned;
 // `folded` ([head][t][kv_rank], nullable) is copied in front of it; `flat_out` ([head][t][dim], nullable) receives
 // the unrotated part.
-int mll_latent_query(const float* q, int n_tokens, int heads, int dim, int rot_dim, int kv_rank, const float* cos_sin,
+int mll_latent_query(const float* q, int64_t q_stride, int n_tokens, int heads, int dim, int rot_dim, int kv_rank, const float* cos_sin,
                      const void* folded, void* flat_out, void* q_full, int dtype, hipStream_t stream);
 
 // out[t][h][o] = sum_i x[t][h][i] * w[h][i][o] (* sigmoid(gate[t][h * n_out + o]) with gate, float32 rows gate_stride
-// apart), sums float32 in ascending i. Strides in elements. Built for (x, w, out) = (f32, f32, f32), (f32, bf16, bf16),
+// apart; with gate_a_head one gate a head: gate[t][h]), sums float32 in ascending i. Strides in elements. Built for (x, w, out) = (f32, f32, f32), (f32, bf16, bf16),
 // (bf16, bf16, bf16), (f32, bf16, f32).
 int mll_head_product(const void* x, int x_dtype, int64_t x_token_stride, int64_t x_head_stride, const void* w, int w_dtype,
                      void* out, int out_dtype, int64_t out_token_stride, int64_t out_head_stride, const float* gate,
-                     int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream);
+                     int64_t gate_stride, int gate_a_head, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream);
 
-// out[t][h * n + c] = in[h][t][c] (* sigmoid(gate[t][h * n + c]) with gate, float32 rows gate_stride apart); in and out in `dtype`.
-int mll_gate_heads(const void* in, const float* gate, int64_t gate_stride, void* out, int dtype, int n_tokens, int heads, int n,
-                   hipStream_t stream);
+// out[t][h * n + c] = in[h][t][c] (* sigmoid(gate[t][h * n + c]) with gate, float32 rows gate_stride apart; with
+// gate_a_head sigmoid(gate[t][h])); in and out in `dtype`.
+int mll_gate_heads(const void* in, const float* gate, int64_t gate_stride, int gate_a_head, void* out, int dtype, int n_tokens,
+                   int heads, int n, hipStream_t stream);
 
 // For every token and head: softmax over the keys j in (p - window, p] (window <= 0: all j <= p) of
 // (q_full[t][h] . pages[slot_j]) * scale, out[t][h] = sum_j weight_j pages[slot_j][:kv_rank]. A token whose
@@ -347,6 +365,29 @@ int mll_latent_attention(const void* q_full, const void* pages, const int32_t* b
                          const int32_t* seq_of_token, const int32_t* positions, void* out, int64_t out_token_stride,
                          int64_t out_head_stride, int dtype, int n_tokens, int heads, int kv_rank, int rot_dim, int page_size,
                          int window, float scale, hipStream_t stream);
+
+// ---- the gated delta rule (csrc/delta_rule.hip) ------------------------------------------------------------------
+
+// Channels: key_heads query heads of key_dim, key_heads key heads of key_dim, heads value heads of value_dim, in this
+// order, at conv_at of proj's rows. u[t][c] = silu(sum_j taps[c][j] * input(t - (n_taps - 1 - j), c)), the input being
+// proj's for the step's tokens of the same request and the request's kept inputs (kept [slot][n_taps - 1][channels],
+// newest last) before them; query and key heads are then divided by sqrt(sum of squares + unit_eps), queries also
+// multiplied by q_factor. gates[t][2 h] = sigmoid(proj[t][beta_at + h]), gates[t][2 h + 1] = exp(-exp(a_log[h]) *
+// softplus(proj[t][step_at + h] + dt_bias[h])). All float32.
+int mll_delta_prepare(const float* proj, int64_t proj_stride, int conv_at, const float* taps, const float* kept,
+                      const int32_t* seq_of_token, const int32_t* cu_tokens, const int32_t* slots, int beta_at, int step_at,
+                      const float* a_log, const float* dt_bias, float* u, float* gates, int n_tokens, int key_heads, int heads,
+                      int key_dim, int value_dim, int n_taps, float q_factor, float unit_eps, hipStream_t stream);
+
+// kept[slot] <- the newest n_taps - 1 rows of proj[.][conv_at ..] of every request, older kept rows before them where
+// the step brought fewer.
+int mll_conv_keep(const float* proj, int64_t proj_stride, int conv_at, float* kept, const int32_t* cu_tokens,
+                  const int32_t* slots, int n_seqs, int channels, int n_taps, hipStream_t stream);
+
+// Per request and head, over the request's tokens in order, with S = state[slot][head] ([key_dim][value_dim], read
+// first, written last): S *= g; c = beta * (v - S^T k); S += k c^T; out[t][head] = S^T q. u and gates as above.
+int mll_delta_scan(const float* u, const float* gates, float* state, const int32_t* cu_tokens, const int32_t* slots, float* out,
+                   int n_seqs, int key_heads, int heads, int key_dim, int value_dim, hipStream_t stream);
 
 // ---- a recurrent block with a gated linear recurrence (csrc/recurrent.hip) ----------------------------------------
 

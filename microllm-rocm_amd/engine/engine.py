@@ -450,6 +450,8 @@ class Engine:
             mix = give = None
             if hasattr(pending, "values") and hasattr(pending, "give"):     # a delta for several streams (parts.streams)
                 pending, mix, give = pending.values, pending.mix, pending.give
+            if hasattr(pending, "resolved"):        # a result that is normed itself before it joins the stream (parts.norm)
+                pending = pending.resolved()
             if isinstance(pending, torch.Tensor):   # else the entry's last product added its result itself
                 delta = pending.to(torch.float32)
                 delta = delta.sum(0) if delta.dim() == 3 else delta

@@ -110,6 +110,61 @@ def rms_norm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch
     return out
 
 
+def rms_norm_after(h: torch.Tensor, delta: torch.Tensor, after_weight: torch.Tensor, after_eps: float, mult: float,
+                   weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                   write_h: bool = False) -> Optional[torch.Tensor]:
+    """``v = h[rows] + mult * rms_norm(delta[rows]) * after_weight`` (``delta`` may be float32 partial sums ``[parts,
+    tokens, width]``, added in order first); with ``write_h`` the sum replaces ``h``; returns ``rms_norm(v) * weight``,
+    or None without ``weight``."""
+    lib = library.load()
+    _device_tensor(h, "residual stream", torch.float32)
+    _device_tensor(after_weight, "norm weight of the delta", torch.float32)
+    _need(h.dim() == 2 and tuple(after_weight.shape) == (h.shape[1],), "the delta's norm weight must match the stream's width")
+    width = h.shape[1]
+    _device_tensor(delta, "delta")
+    _need(delta.dtype in (torch.float32, out_dtype), "delta must be float32 or have the output's dtype")
+    n_partials = 1
+    if delta.dim() == 3:
+        n_partials = delta.shape[0]
+        _need(n_partials >= 1 and tuple(delta.shape[1:]) == tuple(h.shape), "delta parts must have the residual stream's shape")
+    else:
+        _need(tuple(delta.shape) == tuple(h.shape), "delta must have the residual stream's shape")
+    if rows is not None:
+        _device_tensor(rows, "row selection", torch.int32)
+        _need(not write_h, "cannot write h through a row selection")
+        n_rows = rows.shape[0]
+    else:
+        n_rows = h.shape[0]
+    out = None
+    if weight is not None:
+        _device_tensor(weight, "norm weight", torch.float32)
+        _need(tuple(weight.shape) == (width,), "the norm weight must match the stream's width")
+        out = torch.empty((n_rows, width), dtype=out_dtype, device=h.device)
+    _check(lib.mll_rms_norm_after(_ptr(h), _ptr(delta), _code(delta.dtype), n_partials, ctypes.c_int64(h.numel()), _ptr(rows),
+                                  _ptr(after_weight), ctypes.c_float(after_eps), ctypes.c_float(mult), _ptr(weight),
+                                  ctypes.c_float(eps), _ptr(out), _code(out_dtype), n_rows, width, int(write_h), _stream()), lib)
+    return out
+
+
+def add_bias(values: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """``values[..., c] += bias[c]`` in place: float32 ``[rows, width]``, or partial sums ``[parts, rows, width]``, whose
+    first part takes the bias."""
+    lib = library.load()
+    _device_tensor(values, "values", torch.float32)
+    _device_tensor(bias, "bias", torch.float32)
+    _need(values.dim() in (2, 3) and tuple(bias.shape) == (values.shape[-1],), "one bias a column")
+    _check(lib.mll_add_bias(_ptr(values), _ptr(bias), ctypes.c_int64(values.shape[-2]), values.shape[-1], _stream()), lib)
+    return values
+
+
+def softcap(values: torch.Tensor, cap: float) -> torch.Tensor:
+    """``cap * tanh(values / cap)`` in place (float32)."""
+    lib = library.load()
+    _device_tensor(values, "values", torch.float32)
+    _check(lib.mll_softcap(_ptr(values), ctypes.c_int64(values.numel()), ctypes.c_float(cap), _stream()), lib)
+    return values
+
+
 def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     lib = library.load()
     _device_tensor(h, "residual stream", torch.float32)
@@ -1135,17 +1190,37 @@ def _parts_of(tensor: torch.Tensor, name: str) -> Tuple[int, int]:
 def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                   positions: torch.Tensor, slot_mapping: torch.Tensor, temp_coef: float, temp_every: int,
                   k_pages: torch.Tensor, v_pages: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int,
-                  out_dtype: torch.dtype, tiled_page_size: int = 0) -> torch.Tensor:
+                  out_dtype: torch.dtype, tiled_page_size: int = 0, bias: Optional[torch.Tensor] = None,
+                  normed: Optional[bool] = None, queries_only: bool = False) -> torch.Tensor:
     """Norm of queries and keys over their head, the queries' factor by position, keys and values into their pages
     (``[page, position, kv_head, dim]``, or with ``tiled_page_size`` the pages of ``cache.layout`` with that many
-    positions each); returns the queries ``[tokens, heads * key_dim]``."""
+    positions each); returns the queries ``[tokens, heads * key_dim]``. ``bias`` (one number a column of a row) is
+    added first. ``normed`` (by default: where weights are given) divides queries and keys by their root mean square
+    also without weights. With ``queries_only`` the rows hold queries alone and nothing is stored (a layer that
+    reads another's keys and values)."""
     lib = library.load()
     n_parts, part_stride = _parts_of(qkv, "q/k/v")
     n_tokens = qkv.shape[-2]
-    _need(qkv.shape[-1] == (heads + kv_heads) * key_dim + kv_heads * value_dim, "q/k/v rows have the wrong width")
+    row_width = heads * key_dim if queries_only else (heads + kv_heads) * key_dim + kv_heads * value_dim
+    _need(qkv.shape[-1] == row_width, "q/k/v rows have the wrong width")
     _device_tensor(positions, "positions", torch.int32)
+    _need(positions.shape[0] >= n_tokens, "a position for every token")
+    if normed is None:
+        normed = q_weight is not None
+    if bias is not None:
+        _device_tensor(bias, "projection bias", torch.float32)
+        _need(tuple(bias.shape) == (row_width,), "one bias a column of a row")
+    q_out = torch.empty((n_tokens, heads * key_dim), dtype=out_dtype, device=qkv.device)
+    if queries_only:
+        _need(q_weight is None or (q_weight.is_cuda and q_weight.dtype == torch.float32 and tuple(q_weight.shape) == (key_dim,)),
+              "the query norm weight must be float32 of the head's size")
+        _check(lib.mll_qk_norm_store(_ptr(qkv), n_parts, ctypes.c_int64(part_stride), _ptr(q_weight), _ptr(q_weight),
+                                     ctypes.c_float(eps), _ptr(positions), None, ctypes.c_float(temp_coef),
+                                     int(temp_every), _ptr(q_out), None, None, _code(out_dtype), n_tokens,
+                                     heads, kv_heads, key_dim, value_dim, 0, _ptr(bias), int(normed), 1, _stream()), lib)
+        return q_out
     _device_tensor(slot_mapping, "slot mapping", torch.int32)
-    _need(positions.shape[0] >= n_tokens and slot_mapping.shape[0] >= n_tokens, "positions and slots for every token")
+    _need(slot_mapping.shape[0] >= n_tokens, "a slot for every token")
     for name, weight in (("query norm weight", q_weight), ("key norm weight", k_weight)):
         if weight is not None:
             _device_tensor(weight, name, torch.float32)
@@ -1159,20 +1234,22 @@ def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight:
         _need(k_pages.dim() == 4 and tuple(k_pages.shape[2:]) == (kv_heads, key_dim), "key pages are [page, position, kv_head, key_dim]")
         _need(v_pages.dim() == 4 and tuple(v_pages.shape[2:]) == (kv_heads, value_dim) and v_pages.shape[:2] == k_pages.shape[:2],
               "value pages are [page, position, kv_head, value_dim]")
-    q_out = torch.empty((n_tokens, heads * key_dim), dtype=out_dtype, device=qkv.device)
     _check(lib.mll_qk_norm_store(_ptr(qkv), n_parts, ctypes.c_int64(part_stride), _ptr(q_weight), _ptr(k_weight),
                                  ctypes.c_float(eps), _ptr(positions), _ptr(slot_mapping), ctypes.c_float(temp_coef),
                                  int(temp_every), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _code(out_dtype), n_tokens,
-                                 heads, kv_heads, key_dim, value_dim, int(tiled_page_size), _stream()), lib)
+                                 heads, kv_heads, key_dim, value_dim, int(tiled_page_size), _ptr(bias), int(normed), 0,
+                                 _stream()), lib)
     return q_out
 
 
 def bias_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                    seq_of_token: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor],
                    sink: Optional[torch.Tensor], scale: float, out_scale: float, heads: int, kv_heads: int, key_dim: int,
-                   value_dim: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Causal attention with ``bias[min(distance, last row), head]`` added to the scaled scores and ``exp(sink[head])``
-    in the softmax's denominator; ``out`` may be columns of a wider buffer (its row stride is taken)."""
+                   value_dim: int, out: Optional[torch.Tensor] = None, slopes: Optional[torch.Tensor] = None,
+                   window: int = 0) -> torch.Tensor:
+    """Causal attention with ``bias[min(distance, last row), head]`` added to the scaled scores, ``slopes[head] *
+    distance`` taken off them, and ``exp(sink[head])`` in the softmax's denominator; with ``window`` a query sees
+    itself and the ``window - 1`` keys before it; ``out`` may be columns of a wider buffer (its row stride is taken)."""
     lib = library.load()
     _device_tensor(q, "queries")
     n_tokens = q.shape[0]
@@ -1196,6 +1273,10 @@ def bias_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
     if sink is not None:
         _device_tensor(sink, "sink", torch.float32)
         _need(tuple(sink.shape) == (heads,), "one sink a head")
+    if slopes is not None:
+        _device_tensor(slopes, "slopes", torch.float32)
+        _need(tuple(slopes.shape) == (heads,), "one slope a head")
+    _need(window >= 0, "a window is positive, or 0 for none")
     if out is None:
         out = torch.empty((n_tokens, heads * value_dim), dtype=q.dtype, device=q.device)
     _need(out.is_cuda and out.dtype == q.dtype and out.dim() == 2 and tuple(out.shape) == (n_tokens, heads * value_dim)
@@ -1204,7 +1285,7 @@ def bias_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
                                   _ptr(seq_of_token), _ptr(positions), _ptr(bias), longest, _ptr(sink),
                                   ctypes.c_void_p(out.data_ptr()), ctypes.c_int64(out.stride(0) if n_tokens > 1 else max(out.stride(0), heads * value_dim)),
                                   _code(q.dtype), n_tokens, heads, kv_heads, key_dim, value_dim, page_size,
-                                  ctypes.c_float(scale), ctypes.c_float(out_scale), _stream()), lib)
+                                  ctypes.c_float(scale), ctypes.c_float(out_scale), _ptr(slopes), int(window), _stream()), lib)
     return out
 
 
@@ -1272,21 +1353,99 @@ def gla_gate(o: torch.Tensor, proj: torch.Tensor, gate_offset: int, weight: torc
     return out
 
 
+# ---- the gated delta rule ----------------------------------------------------------------------------------------
+def delta_prepare(proj: torch.Tensor, conv_at: int, taps: torch.Tensor, kept: Optional[torch.Tensor], seq_of_token: torch.Tensor,
+                  cu_tokens: torch.Tensor, slots: torch.Tensor, beta_at: int, step_at: int, a_log: torch.Tensor,
+                  dt_bias: torch.Tensor, key_heads: int, heads: int, key_dim: int, value_dim: int, q_factor: float,
+                  unit_eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Queries, keys and values of a step's tokens from the float32 projections ``proj``: a causal convolution per
+    channel over ``proj[:, conv_at:conv_at + channels]`` (``taps`` ``[channels, n_taps]``, the last column the token's
+    own; before the step's first token the request's ``kept`` inputs ``[slots, n_taps - 1, channels]``), SiLU, unit
+    vectors per query and key head, the queries times ``q_factor``; and per head ``beta = sigmoid(proj[:, beta_at +
+    h])`` and ``g = exp(-exp(a_log[h]) * softplus(proj[:, step_at + h] + dt_bias[h]))``. Returns ``u`` ``[tokens,
+    channels]`` (queries, keys, values) and ``gates`` ``[tokens, heads, 2]``, float32."""
+    lib = library.load()
+    _device_tensor(proj, "projections", torch.float32)
+    _device_tensor(taps, "convolution taps", torch.float32)
+    channels = 2 * key_heads * key_dim + heads * value_dim
+    _need(proj.dim() == 2 and taps.dim() == 2 and taps.shape[0] == channels, "taps are [channels, n_taps]")
+    n_taps = taps.shape[1]
+    n_tokens = proj.shape[0]
+    _need(0 <= conv_at and conv_at + channels <= proj.shape[1] and 0 <= beta_at and beta_at + heads <= proj.shape[1]
+          and 0 <= step_at and step_at + heads <= proj.shape[1], "the columns lie outside the projections' rows")
+    if n_taps > 1:
+        _device_tensor(kept, "kept inputs", torch.float32)
+        _need(kept.dim() == 3 and tuple(kept.shape[1:]) == (n_taps - 1, channels), "kept inputs are [slots, n_taps - 1, channels]")
+    for name, tensor in (("A_log", a_log), ("dt_bias", dt_bias)):
+        _device_tensor(tensor, name, torch.float32)
+        _need(tuple(tensor.shape) == (heads,), f"{name} holds one number a head")
+    _device_tensor(seq_of_token, "request of every token", torch.int32)
+    _device_tensor(cu_tokens, "token offsets", torch.int32)
+    _device_tensor(slots, "state slots", torch.int32)
+    _need(seq_of_token.shape[0] >= n_tokens, "a request for every token")
+    u = torch.empty((n_tokens, channels), dtype=torch.float32, device=proj.device)
+    gates = torch.empty((n_tokens, heads, 2), dtype=torch.float32, device=proj.device)
+    _check(lib.mll_delta_prepare(_ptr(proj), ctypes.c_int64(proj.shape[1]), conv_at, _ptr(taps), _ptr(kept if n_taps > 1 else None),
+                                 _ptr(seq_of_token), _ptr(cu_tokens), _ptr(slots), beta_at, step_at, _ptr(a_log), _ptr(dt_bias),
+                                 _ptr(u), _ptr(gates), n_tokens, key_heads, heads, key_dim, value_dim, n_taps,
+                                 ctypes.c_float(q_factor), ctypes.c_float(unit_eps), _stream()), lib)
+    return u, gates
+
+
+def conv_keep(proj: torch.Tensor, conv_at: int, kept: torch.Tensor, cu_tokens: torch.Tensor, slots: torch.Tensor, n_seqs: int) -> None:
+    """``kept`` ``[slots, n_taps - 1, channels]`` receives every request's newest inputs ``proj[:, conv_at:conv_at +
+    channels]`` of the step, older kept ones before them where the step brought fewer than ``n_taps - 1``."""
+    lib = library.load()
+    _device_tensor(proj, "projections", torch.float32)
+    _device_tensor(kept, "kept inputs", torch.float32)
+    _need(proj.dim() == 2 and kept.dim() == 3, "projections [tokens, columns] and kept inputs [slots, n_taps - 1, channels]")
+    channels, n_taps = kept.shape[2], kept.shape[1] + 1
+    _need(0 <= conv_at and conv_at + channels <= proj.shape[1], "the convolution's columns lie outside the projections' rows")
+    _device_tensor(cu_tokens, "token offsets", torch.int32)
+    _device_tensor(slots, "state slots", torch.int32)
+    _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
+    _check(lib.mll_conv_keep(_ptr(proj), ctypes.c_int64(proj.shape[1]), conv_at, _ptr(kept), _ptr(cu_tokens), _ptr(slots), n_seqs,
+                             channels, n_taps, _stream()), lib)
+
+
+def delta_scan(u: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, cu_tokens: torch.Tensor, slots: torch.Tensor,
+               n_seqs: int, key_heads: int, heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
+    """The delta rule over every request's tokens of the step, in order: ``S *= g; c = beta (v - S^T k); S += k c^T;
+    o = S^T q`` with ``S = state[slot, head]`` (``[slots, heads, key_dim, value_dim]`` float32, read first and written
+    last). ``u`` and ``gates`` as ``delta_prepare`` returns them. Returns ``[tokens, heads * value_dim]`` float32."""
+    lib = library.load()
+    _device_tensor(u, "queries, keys and values", torch.float32)
+    _device_tensor(gates, "gates", torch.float32)
+    _device_tensor(state, "state", torch.float32)
+    _device_tensor(cu_tokens, "token offsets", torch.int32)
+    _device_tensor(slots, "state slots", torch.int32)
+    n_tokens = u.shape[0]
+    _need(u.dim() == 2 and u.shape[1] == 2 * key_heads * key_dim + heads * value_dim, "u is [tokens, queries | keys | values]")
+    _need(tuple(gates.shape) == (n_tokens, heads, 2), "gates are [tokens, heads, 2]")
+    _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, key_dim, value_dim), "state is [slots, heads, key_dim, value_dim]")
+    _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
+    out = torch.empty((n_tokens, heads * value_dim), dtype=torch.float32, device=u.device)
+    _check(lib.mll_delta_scan(_ptr(u), _ptr(gates), _ptr(state), _ptr(cu_tokens), _ptr(slots), _ptr(out), n_seqs, key_heads, heads,
+                              key_dim, value_dim, _stream()), lib)
+    return out
+
+
 # ---- attention through latents -----------------------------------------------------------------------------------
-def latent_prepare(proj: torch.Tensor, q_at: int, q_rank: int, q_weight: torch.Tensor, kv_at: int, kv_rank: int, rot_dim: int,
+def latent_prepare(proj: torch.Tensor, q_at: int, q_rank: int, q_weight: Optional[torch.Tensor], kv_at: int, kv_rank: int, rot_dim: int,
                    kv_weight: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
                    slot_mapping: Optional[torch.Tensor], out_dtype: torch.dtype, pages: Optional[torch.Tensor] = None,
                    k_pages: Optional[torch.Tensor] = None, v_pages: Optional[torch.Tensor] = None,
-                   tiled_page_size: int = 0) -> torch.Tensor:
+                   tiled_page_size: int = 0) -> Optional[torch.Tensor]:
     """The norms of a token's two latents from its float32 down projections ``proj`` ``[tokens, columns]``; returns the
-    queries' normed latent ``[tokens, q_rank]``. With ``slot_mapping`` the keys' normed latent and the turned key
+    queries' normed latent ``[tokens, q_rank]`` (``q_rank`` 0: the queries have no latent, and None comes back). With ``slot_mapping`` the keys' normed latent and the turned key
     part go into ``pages`` ``[page, position, kv_rank + rot_dim]`` or, with ``tiled_page_size``, into key and value
     pages of ``cache.layout`` (one kv head of ``kv_rank + rot_dim`` dims, the same row in both)."""
     lib = library.load()
     _device_tensor(proj, "down projections", torch.float32)
     _need(proj.dim() == 2 and 0 <= q_at and q_at + q_rank <= proj.shape[1], "the queries' latent lies outside the projections' rows")
-    _device_tensor(q_weight, "query latent norm weight", torch.float32)
-    _need(tuple(q_weight.shape) == (q_rank,), "the queries' norm weight must match their latent")
+    if q_rank:
+        _device_tensor(q_weight, "query latent norm weight", torch.float32)
+        _need(tuple(q_weight.shape) == (q_rank,), "the queries' norm weight must match their latent")
     n_tokens = proj.shape[0]
     if slot_mapping is not None:
         _need(0 <= kv_at and kv_at + kv_rank + rot_dim <= proj.shape[1], "the keys' latent lies outside the projections' rows")
@@ -1300,8 +1459,8 @@ def latent_prepare(proj: torch.Tensor, q_at: int, q_rank: int, q_weight: torch.T
         else:
             _device_tensor(pages, "latent pages", out_dtype)
             _need(pages.dim() == 3 and pages.shape[2] == kv_rank + rot_dim, "latent pages are [page, position, kv_rank + rot_dim]")
-    q_latent = torch.empty((n_tokens, q_rank), dtype=out_dtype, device=proj.device)
-    _check(lib.mll_latent_prepare(_ptr(proj), ctypes.c_int64(proj.shape[1]), q_at, q_rank, _ptr(q_weight), kv_at, kv_rank, rot_dim,
+    q_latent = torch.empty((n_tokens, q_rank), dtype=out_dtype, device=proj.device) if q_rank else None
+    _check(lib.mll_latent_prepare(_ptr(proj), ctypes.c_int64(proj.shape[1]), q_at, q_rank, _ptr(q_weight if q_rank else None), kv_at, kv_rank, rot_dim,
                                   _ptr(kv_weight), ctypes.c_float(eps), _ptr(cos_sin), _ptr(slot_mapping), _ptr(q_latent),
                                   _ptr(pages), _ptr(k_pages), _ptr(v_pages), int(tiled_page_size), _code(out_dtype), n_tokens,
                                   _stream()), lib)
@@ -1310,13 +1469,14 @@ def latent_prepare(proj: torch.Tensor, q_at: int, q_rank: int, q_weight: torch.T
 
 def latent_query(q: torch.Tensor, heads: int, dim: int, rot_dim: int, kv_rank: int, cos_sin: torch.Tensor, q_full: torch.Tensor,
                  folded: Optional[torch.Tensor] = None, want_flat: bool = False) -> Optional[torch.Tensor]:
-    """``q`` float32 ``[tokens, heads * (dim + rot_dim)]``: the turned rotated parts go behind the folded parts in
+    """``q`` float32 ``[tokens, heads * (dim + rot_dim)]`` (may be columns of wider rows): the turned rotated parts go behind the folded parts in
     ``q_full`` ``[tokens, heads * (kv_rank + rot_dim)]``; ``folded`` ``[heads, tokens, kv_rank]`` is copied in front;
     with ``want_flat`` the unrotated parts are returned as ``[heads, tokens, dim]`` in ``q_full``'s dtype."""
     lib = library.load()
-    _device_tensor(q, "queries", torch.float32)
+    _need(q.is_cuda and q.dtype == torch.float32 and q.dim() == 2 and q.stride(1) == 1, "queries are float32 rows with unit column stride")
     n_tokens = q.shape[0]
-    _need(q.dim() == 2 and q.shape[1] == heads * (dim + rot_dim), "queries are [tokens, heads * (dim + rot_dim)]")
+    _need(q.shape[1] == heads * (dim + rot_dim), "queries are [tokens, heads * (dim + rot_dim)]")
+    q_stride = max(q.stride(0), q.shape[1])
     _device_tensor(cos_sin, "cos/sin table", torch.float32)
     _need(tuple(cos_sin.shape) == (n_tokens, rot_dim // 2, 2) and rot_dim % 2 == 0, "the cos/sin table must be [tokens, rot_dim / 2, 2]")
     _device_tensor(q_full, "folded queries")
@@ -1325,7 +1485,7 @@ def latent_query(q: torch.Tensor, heads: int, dim: int, rot_dim: int, kv_rank: i
         _device_tensor(folded, "folded parts", q_full.dtype)
         _need(tuple(folded.shape) == (heads, n_tokens, kv_rank), "folded parts are [heads, tokens, kv_rank]")
     flat = torch.empty((heads, n_tokens, dim), dtype=q_full.dtype, device=q.device) if want_flat else None
-    _check(lib.mll_latent_query(_ptr(q), n_tokens, heads, dim, rot_dim, kv_rank, _ptr(cos_sin), _ptr(folded), _ptr(flat), _ptr(q_full),
+    _check(lib.mll_latent_query(_ptr(q), ctypes.c_int64(q_stride), n_tokens, heads, dim, rot_dim, kv_rank, _ptr(cos_sin), _ptr(folded), _ptr(flat), _ptr(q_full),
                                 _code(q_full.dtype), _stream()), lib)
     return flat
 
@@ -1334,9 +1494,10 @@ HEAD_PRODUCT_TYPES = {(torch.float32, torch.float32, torch.float32), (torch.floa
                       (torch.bfloat16, torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16, torch.float32)}
 
 
-def head_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+def head_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None,
+                 gate_a_head: bool = False) -> torch.Tensor:
     """``out[t, h, o] = sum_i x[t, h, i] * weight[h, i, o]``, times ``sigmoid(gate[t, h * n_out + o])`` with ``gate``
-    (float32 rows). ``x`` ``[tokens, heads, n_in]`` and ``out`` ``[tokens, heads, n_out]`` may be views with strides of
+    (float32 rows), or times ``sigmoid(gate[t, h])`` with ``gate_a_head``. ``x`` ``[tokens, heads, n_in]`` and ``out`` ``[tokens, heads, n_out]`` may be views with strides of
     their own over tokens and heads (unit stride along the last axis); the weight is contiguous."""
     lib = library.load()
     _device_tensor(weight, "per-head weight")
@@ -1348,32 +1509,33 @@ def head_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, gate:
     _need((x.dtype, weight.dtype, out.dtype) in HEAD_PRODUCT_TYPES, f"head_product is not built for {x.dtype}, {weight.dtype}, {out.dtype}")
     gate_stride = 0
     if gate is not None:
-        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape == (n_tokens, heads * n_out) and gate.stride(1) == 1,
-              "the gate is float32 [tokens, heads * n_out] with unit column stride")
+        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and gate.stride(1) == 1
+              and gate.shape == (n_tokens, heads if gate_a_head else heads * n_out),
+              "the gate is float32 [tokens, heads * n_out] (or [tokens, heads]) with unit column stride")
         gate_stride = gate.stride(0)
     _check(lib.mll_head_product(ctypes.c_void_p(x.data_ptr()), _code(x.dtype), ctypes.c_int64(x.stride(0)), ctypes.c_int64(x.stride(1)),
                                 _ptr(weight), _code(weight.dtype), ctypes.c_void_p(out.data_ptr()), _code(out.dtype),
                                 ctypes.c_int64(out.stride(0)), ctypes.c_int64(out.stride(1)),
                                 ctypes.c_void_p(gate.data_ptr() if gate is not None else 0), ctypes.c_int64(gate_stride),
-                                n_tokens, heads, n_in, n_out, _stream()), lib)
+                                int(gate_a_head), n_tokens, heads, n_in, n_out, _stream()), lib)
     return out
 
 
-def gate_heads(values: torch.Tensor, gate: Optional[torch.Tensor]) -> torch.Tensor:
+def gate_heads(values: torch.Tensor, gate: Optional[torch.Tensor], gate_a_head: bool = False) -> torch.Tensor:
     """``[heads, tokens, n]`` (a batched product's result) -> ``[tokens, heads * n]``, times ``sigmoid(gate)`` (float32
-    ``[tokens, heads * n]``, unit column stride) if given."""
+    ``[tokens, heads * n]``, or ``[tokens, heads]`` with ``gate_a_head``; unit column stride) if given."""
     lib = library.load()
     _device_tensor(values, "values per head")
     _need(values.dim() == 3, "values are [heads, tokens, n]")
     heads, n_tokens, n = values.shape
     gate_stride = 0
     if gate is not None:
-        _need(gate.is_cuda and gate.dtype == torch.float32 and tuple(gate.shape) == (n_tokens, heads * n) and gate.stride(1) == 1,
-              "the gate is float32 [tokens, heads * n] with unit column stride")
+        _need(gate.is_cuda and gate.dtype == torch.float32 and tuple(gate.shape) == (n_tokens, heads if gate_a_head else heads * n)
+              and gate.stride(1) == 1, "the gate is float32 [tokens, heads * n] (or [tokens, heads]) with unit column stride")
         gate_stride = gate.stride(0)
     out = torch.empty((n_tokens, heads * n), dtype=values.dtype, device=values.device)
     _check(lib.mll_gate_heads(_ptr(values), ctypes.c_void_p(gate.data_ptr() if gate is not None else 0), ctypes.c_int64(gate_stride),
-                              _ptr(out), _code(values.dtype), n_tokens, heads, n, _stream()), lib)
+                              int(gate_a_head), _ptr(out), _code(values.dtype), n_tokens, heads, n, _stream()), lib)
     return out
 
 

@@ -1,4 +1,4 @@
-from . import (attention, bias_attention, block, experts, feedforward, latent_attention, linear_attention, model, norm, parallel, position,
+from . import (attention, bias_attention, block, delta_rule, experts, feedforward, latent_attention, linear_attention, model, norm, parallel, position,
                recurrent, streams)  # noqa: F401  (register the built-in kinds)
 from .base import (CacheNeed, CompositeNeed, PagedKeyValueNeed, PagedLatentNeed, FeedForward, INT_TABLE, MATRIX, Mixer, Norm, PagedKVNeed, Part, PositionEncoding, Runtime,
                    StateNeed, TensorDecl, VECTOR)

@@ -1,16 +1,23 @@
-"""Causal softmax attention whose positions enter through the scores: a learned bias by distance bucket, a sink in
-the softmax, and a query factor that grows with the position. No rotation.
+"""Causal softmax attention whose positions enter through the scores: a learned bias by distance bucket or a slope a
+head times the distance, a sink in the softmax, a query factor that grows with the position, a sliding window. No
+rotation.
 
-``q = Wq x``, ``k = Wk x``, ``v = Wv x`` (no biases); query head ``h`` uses kv head ``h // (heads / kv_heads)``; keys
+``q = Wq x``, ``k = Wk x``, ``v = Wv x`` (with ``projection_bias`` each and the output projection have a bias, named
+as the weight with ``_bias``); query head ``h`` uses kv head ``h // (heads / kv_heads)``; keys
 have ``key_dim`` and values ``value_dim`` channels. With ``qk_norm`` queries and keys are divided by their root mean
-square over the head (eps inside the root) and multiplied by a weight ``[key_dim]`` that all heads share. Queries
+square over the head (eps inside the root) and, unless ``qk_norm_weight`` is false, multiplied by a weight
+``[key_dim]`` that all heads share. Queries
 at position ``p`` are multiplied by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)``. The score of key ``j``
 for a query at ``i >= j`` is ``(q . k) * scale + table[bucket(i - j), h]`` with, for a table of ``B`` rows and a
 longest distance ``D``: ``bucket(n) = n`` below ``B / 2``, else ``min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(D / (B/2))
-* (B - B/2)))``. The softmax's denominator also holds ``exp(sink[h])``, which has no key and no value.
+* (B - B/2)))``. With ``slopes`` (one number a head) ``slopes[h] * (i - j)`` is taken off the score instead. The
+softmax's denominator also holds ``exp(sink[h])``, which has no key and no value. With ``window`` a query sees
+``0 <= i - j < window``. With ``owns_kv`` false the layer has no ``Wk`` and ``Wv``: it reads the keys (as cached, after
+their norm) and values of another run entry, with queries, bias and window of its own.
 
 Every distance from ``D`` on falls into the last bucket, so the table is unrolled once, at load, into one row per
-distance up to ``D`` and the kernels index it with ``min(i - j, D)``.
+distance up to ``D`` and the kernels index it with ``min(i - j, D)``. Slopes under a window become such a table for
+the MFMA kernels (a row per distance inside the window); the kernel for plain pages takes the slopes themselves.
 
 In bfloat16, with keys and values of one width that is a multiple of 16, the pages are the paged attention's own
 (``PagedKVNeed``) and the attention runs on its MFMA kernels, which take the bias, the sink and the result's factor
@@ -60,14 +67,28 @@ class BucketBiasAttention(Mixer):
         self.bias_rows = int(p["bias_rows"]) if p.get("bias_rows") else 0      # 0: no bias
         self.bias_max = int(p.get("bias_max", 0))
         self.has_sink = bool(p.get("sink", True))
+        self.projection_bias = bool(p.get("projection_bias", False))
+        self.qk_norm_weight = bool(p.get("qk_norm_weight", True)) and self.qk_norm
+        self.slope_values = [float(value) for value in p["slopes"]] if p.get("slopes") is not None else None
+        self.window = int(p["window"]) if p.get("window") else 0
+        # how long the keys and values are kept: the widest window of the layers that read them (0: for ever)
+        self.kept_window = int(p.get("kept_window") or self.window) if self.window else 0
+        self.owns_kv = bool(p.get("owns_kv", True))
         if self.heads % self.kv_heads != 0:
             raise ValueError("heads must divide into kv_heads groups")
         if self.bias_rows and self.bias_max <= self.bias_rows // 2:
             raise ValueError("bias_max must lie beyond the distances that have a bucket of their own")
-        # the paged attention's pages and MFMA kernels, where they fit (the bias column must fit the prefill kernel's LDS)
-        self.tiled = (runtime.dtype == torch.bfloat16 and self.key_dim == self.value_dim and self.key_dim % 16 == 0
-                      and self.key_dim <= 256 and self.bias_max + 1 <= kernels.MFMA_BIAS_ROWS)
-        self.planner = QueryTilePlanner(False) if self.tiled else None
+        if self.slope_values is not None and (len(self.slope_values) != self.heads or self.bias_rows):
+            raise ValueError("one slope a head, and either slopes or a table of buckets")
+        if self.window and self.kept_window < self.window:
+            raise ValueError("the keys and values must be kept at least as long as this layer's window")
+        # the paged attention's pages and MFMA kernels, where they fit (the bias column must fit the prefill kernel's LDS;
+        # slopes are such a column only under a window that fits)
+        table_rows = self.window if self.slope_values is not None else self.bias_max + 1
+        self.tiled = (bool(p.get("mfma", True)) and runtime.dtype == torch.bfloat16 and self.key_dim == self.value_dim
+                      and self.key_dim % 16 == 0 and self.key_dim <= 256 and 0 < table_rows <= kernels.MFMA_BIAS_ROWS)
+        self.planner = QueryTilePlanner(bool(self.window)) if self.tiled else None
+        self.slopes = self.o_bias = self.qkv_bias = None
         self.qkv_weight: Optional[Weight] = None
         self.o_tensor: Optional[torch.Tensor] = None
         self.o_weight: Optional[Weight] = None
@@ -79,27 +100,46 @@ class BucketBiasAttention(Mixer):
 
     def tensors(self) -> Dict[str, TensorDecl]:
         decls = {self.name("q"): TensorDecl((self.heads * self.key_dim, self.hidden), MATRIX),
-                 self.name("k"): TensorDecl((self.kv_heads * self.key_dim, self.hidden), MATRIX),
-                 self.name("v"): TensorDecl((self.kv_heads * self.value_dim, self.hidden), MATRIX),
                  self.name("o"): TensorDecl((self.hidden, self.heads * self.value_dim), MATRIX)}
-        if self.qk_norm:
+        if self.owns_kv:
+            decls[self.name("k")] = TensorDecl((self.kv_heads * self.key_dim, self.hidden), MATRIX)
+            decls[self.name("v")] = TensorDecl((self.kv_heads * self.value_dim, self.hidden), MATRIX)
+        if self.projection_bias:
+            for role in self._in_roles() + ("o",):
+                decls[self.name(f"{role}_bias")] = TensorDecl((decls[self.name(role)].shape[0],), VECTOR)
+        if self.qk_norm_weight:
             decls[self.name("q_norm")] = TensorDecl((self.key_dim,), VECTOR)
-            decls[self.name("k_norm")] = TensorDecl((self.key_dim,), VECTOR)
+            if self.owns_kv:
+                decls[self.name("k_norm")] = TensorDecl((self.key_dim,), VECTOR)
         if self.bias_rows:
             decls[self.name("bias")] = TensorDecl((self.bias_rows, self.heads), VECTOR)
         if self.has_sink:
             decls[self.name("sink")] = TensorDecl((self.heads,), VECTOR)
         return decls
 
+    def _in_roles(self):
+        return ("q", "k", "v") if self.owns_kv else ("q",)
+
     def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        weights = [tensors[self.name(role)] for role in ("q", "k", "v")]
+        weights = [tensors[self.name(role)] for role in self._in_roles()]
         if len({w.dtype for w in weights}) != 1:
             raise TypeError("the q, k and v weights of one layer must share a dtype to be stacked")
-        self.qkv_weight = Weight(torch.cat(weights, dim=0).contiguous(), keep_plain=self.runtime.keep_plain_weights)
+        self.qkv_weight = Weight(torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0],
+                                 keep_plain=self.runtime.keep_plain_weights)
         del weights
         self.o_tensor = tensors[self.name("o")]
-        if self.qk_norm:
-            self.q_norm, self.k_norm = tensors[self.name("q_norm")], tensors[self.name("k_norm")]
+        if self.projection_bias:
+            self.qkv_bias = torch.cat([tensors[self.name(f"{role}_bias")] for role in self._in_roles()]).contiguous()
+            self.o_bias = tensors[self.name("o_bias")]
+        if self.qk_norm_weight:
+            self.q_norm = tensors[self.name("q_norm")]
+            self.k_norm = tensors[self.name("k_norm")] if self.owns_kv else None
+        if self.slope_values is not None:
+            device = self.o_tensor.device
+            self.slopes = torch.tensor(self.slope_values, dtype=torch.float32, device=device)
+            if self.tiled:      # a row per distance inside the window: what lies further is not seen
+                distances = torch.arange(self.window, dtype=torch.float32, device=device)
+                self.bias = (-(distances[:, None] * self.slopes[None, :])).contiguous()
         if self.bias_rows:
             table = tensors[self.name("bias")]
             rows = [distance_bucket(distance, self.bias_rows, self.bias_max) for distance in range(self.bias_max + 1)]
@@ -117,13 +157,17 @@ class BucketBiasAttention(Mixer):
         return self.planner
 
     def cache_need(self):
+        if not self.owns_kv:
+            return None
+        window = self.kept_window or None
         if self.tiled:
-            return PagedKVNeed(self.kv_heads, self.key_dim)
-        return PagedKeyValueNeed(self.kv_heads, self.key_dim, self.value_dim)
+            return PagedKVNeed(self.kv_heads, self.key_dim, window)
+        return PagedKeyValueNeed(self.kv_heads, self.key_dim, self.value_dim, window)
 
     def flops(self, tokens: int) -> float:
-        pairs = tokens * (tokens + 1) / 2
-        columns = (self.heads + self.kv_heads) * self.key_dim + self.kv_heads * self.value_dim
+        window = self.window or tokens
+        pairs = sum(min(position + 1, window) for position in range(tokens))
+        columns = self.heads * self.key_dim + ((self.key_dim + self.value_dim) * self.kv_heads if self.owns_kv else 0)
         if self.o_tensor is not None or self.o_weight is not None:      # else the mixer that took the projection counts it
             columns += self.heads * self.value_dim
         return 2.0 * tokens * self.hidden * columns + 2.0 * self.heads * (self.key_dim + self.value_dim) * pairs
@@ -135,23 +179,25 @@ class BucketBiasAttention(Mixer):
         qkv = linear(x, self.qkv_weight, out_dtype=torch.float32, partials=True)     # rounded once, after norm and factor
         q = kernels.qk_norm_store(qkv, self.q_norm, self.k_norm, self.eps, ctx.positions, view.slot_mapping, self.temp_coef,
                                   self.temp_every, cache.k, cache.v, self.heads, self.kv_heads, self.key_dim, self.value_dim,
-                                  self.runtime.dtype, tiled_page_size=view.page_size if self.tiled else 0)
+                                  self.runtime.dtype, tiled_page_size=view.page_size if self.tiled else 0, bias=self.qkv_bias,
+                                  normed=self.qk_norm, queries_only=not self.owns_kv)
         if self.tiled:
             if out is None:
                 out = torch.empty((x.shape[0], self.heads * self.value_dim), dtype=self.runtime.dtype, device=x.device)
             extras = kernels.AttentionExtras(self.bias, self.sink, out_scale)
-            return kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, 0, self.heads, self.kv_heads, self.key_dim,
-                                           planner=self.planner, extras=extras, out=out)
+            return kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, self.window, self.heads, self.kv_heads,
+                                           self.key_dim, planner=self.planner, extras=extras, out=out)
         return kernels.bias_attention(q, cache.k, cache.v, view.block_table, ctx.seq_of_token, ctx.positions, self.bias,
                                       self.sink, self.scale, out_scale, self.heads, self.kv_heads, self.key_dim,
-                                      self.value_dim, out=out)
+                                      self.value_dim, out=out, slopes=self.slopes, window=self.window)
 
     def forward(self, x, ctx, cache):
         if self.o_weight is None:
             if self.o_tensor is None:
                 raise RuntimeError("this attention's output projection was taken by the mixer it is a part of")
             self.o_weight = Weight(self.take_output_projection(), keep_plain=self.runtime.keep_plain_weights)
-        return linear(self.forward_inner(x, ctx, cache), self.o_weight, out_dtype=torch.float32, partials=True)
+        y = linear(self.forward_inner(x, ctx, cache), self.o_weight, out_dtype=torch.float32, partials=True)
+        return kernels.add_bias(y, self.o_bias) if self.o_bias is not None else y
 
 
 register_part("mixer", "bucket_bias_attention", BucketBiasAttention)

@@ -18,6 +18,7 @@ import torch
 
 from .base import Part, Runtime, TensorDecl
 from .linear import Residual, UnscaledRows
+from .norm import NormedDelta
 from .registry import build_part, register_part
 from .spec import LayerSpec
 
@@ -86,7 +87,38 @@ class PreNormBlock(Block):
         return self.ffn.forward(x, ctx, residual=residual) if residual is not None else self.ffn.forward(x, ctx)
 
 
-_ARRANGEMENTS = {"pre_norm": PreNormBlock}
+class SandwichNormBlock(Block):
+    """A norm before and a norm after each sublayer, and a factor on what joins the stream:
+    ``h' = h + m * NormA(Mixer(Norm1(h)))``, ``h'' = h' + m * NormB(FFN(Norm2(h')))``. The norms after are RMS norms
+    named ``mixer_after`` and ``ffn_after`` in ``LayerSpec.extra``; ``m`` is ``LayerSpec.params["residual_mult"]``
+    (1 if absent). A sublayer's result is handed on as a ``NormedDelta``: the norm that reads the stream next norms
+    and adds it in the same kernel, so no product adds into the stream itself here."""
+
+    def __init__(self, spec: LayerSpec, runtime: Runtime):
+        super().__init__(spec, runtime)
+        self.mult = float(spec.params.get("residual_mult", 1.0))
+        self.mixer_after = self.extra["mixer_after"]
+        self.ffn_after = self.extra.get("ffn_after")
+        if (self.ffn is None) != (self.ffn_after is None):
+            raise ValueError("a feed-forward and the norm after it come together")
+
+    def _normed(self, values, norm) -> NormedDelta:
+        pieces = norm.weight_then_factor()
+        if pieces is None:
+            raise TypeError("the norm after a sublayer must be an RMS norm with a float32 weight")
+        weight, _, eps = pieces
+        return NormedDelta(values, weight, eps, self.mult)
+
+    def forward(self, h, pending, ctx, cache, next_block=None):
+        x = pending if isinstance(pending, UnscaledRows) else self.mixer_norm.forward(h, delta=pending, write_h=True)
+        mixed = self._normed(self.mixer.forward(x, ctx, cache), self.mixer_after)
+        if self.ffn is None:
+            return mixed
+        x = self.ffn_norm.forward(h, delta=mixed, write_h=True)
+        return self._normed(self.ffn.forward(x, ctx), self.ffn_after)
+
+
+_ARRANGEMENTS = {"pre_norm": PreNormBlock, "sandwich_norm": SandwichNormBlock}
 
 
 def register_arrangement(name: str, block_class, replace: bool = False) -> None:

@@ -6,7 +6,9 @@ latent ``c``; the last ``rot_dim``, turned by the token's position, are one key 
 norms are RMS norms with a plain weight. Head ``h`` has keys ``Wuk_h c`` and values ``Wuv_h c``; a query at ``p`` sees
 the keys ``j`` with ``0 <= p - j < window``, scores are ``(q_flat . Wuk_h c_j + q_rot . kr_j) * scale``, the softmax
 is the ordinary one, the heads side by side are multiplied by ``sigmoid(Wg x)`` (``output_gate``) and projected by
-``Wo``. A layer with ``owns_kv`` False has no ``Wdkv``: it reads the latents another run entry cached.
+``Wo``. A layer with ``owns_kv`` False has no ``Wdkv``: it reads the latents another run entry cached. Without a
+``q_rank`` the queries have no latent: ``q = Wq x``. With ``gate_a_head`` the gate is one number a head, ``Wg`` being
+``[heads, hidden]``.
 
 Only ``[c | kr]`` is cached, one row a token. The up projections are folded into the query and into the result:
 ``q'_h = Wuk_h^T q_flat`` (``kv_rank`` numbers) and ``o_h = Wuv_h sum_j p_j c_j``, so the attention has a single kv
@@ -44,7 +46,7 @@ class LatentAttention(Mixer):
         self.dim = int(p["dim"])
         self.rot_dim = int(p["rot_dim"])
         self.vdim = int(p["vdim"])
-        self.q_rank = int(p["q_rank"])
+        self.q_rank = int(p["q_rank"]) if p.get("q_rank") else 0       # 0: queries straight from the input
         self.kv_rank = int(p["kv_rank"])
         self.scale = float(p["scale"])
         self.window = int(p["window"]) if p.get("window") else 0
@@ -53,6 +55,7 @@ class LatentAttention(Mixer):
         self.eps = float(p.get("eps", 1e-6))
         self.owns_kv = bool(p.get("owns_kv", True))
         self.output_gate = bool(p.get("output_gate", False))
+        self.gate_a_head = bool(p.get("gate_a_head", False))
         if self.window and self.kept_window < self.window:
             raise ValueError("the cached rows must be kept at least as long as this layer's window")
         self.position = build_part("position", p["position"], runtime)
@@ -61,9 +64,11 @@ class LatentAttention(Mixer):
         self.row = self.kv_rank + self.rot_dim
         self.tiled = bool(p.get("mfma", True)) and runtime.dtype == torch.bfloat16 and self.row % 16 == 0 and self.row <= 256
         self.planner = QueryTilePlanner(bool(self.window)) if self.tiled else None
+        self.q_width = self.heads * (self.dim + self.rot_dim)
+        self.gate_width = (self.heads if self.gate_a_head else self.heads * self.vdim) if self.output_gate else 0
         self.q_at = 0
-        self.kv_at = self.q_rank
-        self.gate_at = self.q_rank + (self.row if self.owns_kv else 0)
+        self.kv_at = self.q_rank or self.q_width
+        self.gate_at = self.kv_at + (self.row if self.owns_kv else 0)
         self.in_weight: Optional[Weight] = None
         self.uq_weight: Optional[Weight] = None
         self.o_weight: Optional[Weight] = None
@@ -71,30 +76,34 @@ class LatentAttention(Mixer):
 
     def tensors(self) -> Dict[str, TensorDecl]:
         inner = self.heads * self.vdim
-        decls = {self.name("dq"): TensorDecl((self.q_rank, self.hidden), MATRIX),
-                 self.name("dq_norm"): TensorDecl((self.q_rank,), VECTOR),
-                 self.name("uq"): TensorDecl((self.heads * (self.dim + self.rot_dim), self.q_rank), MATRIX),
-                 self.name("uk"): TensorDecl((self.heads * self.dim, self.kv_rank), MATRIX),
+        decls = {self.name("uk"): TensorDecl((self.heads * self.dim, self.kv_rank), MATRIX),
                  self.name("uv"): TensorDecl((inner, self.kv_rank), MATRIX),
                  self.name("o"): TensorDecl((self.hidden, inner), MATRIX)}
+        if self.q_rank:
+            decls[self.name("dq")] = TensorDecl((self.q_rank, self.hidden), MATRIX)
+            decls[self.name("dq_norm")] = TensorDecl((self.q_rank,), VECTOR)
+            decls[self.name("uq")] = TensorDecl((self.q_width, self.q_rank), MATRIX)
+        else:
+            decls[self.name("q")] = TensorDecl((self.q_width, self.hidden), MATRIX)
         if self.owns_kv:
             decls[self.name("dkv")] = TensorDecl((self.row, self.hidden), MATRIX)
             decls[self.name("dkv_norm")] = TensorDecl((self.kv_rank,), VECTOR)
         if self.output_gate:
-            decls[self.name("g")] = TensorDecl((inner, self.hidden), MATRIX)
+            decls[self.name("g")] = TensorDecl((self.gate_width, self.hidden), MATRIX)
         return decls
 
     def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        roles = ["dq"] + (["dkv"] if self.owns_kv else []) + (["g"] if self.output_gate else [])
+        roles = ["dq" if self.q_rank else "q"] + (["dkv"] if self.owns_kv else []) + (["g"] if self.output_gate else [])
         weights = [tensors[self.name(role)] for role in roles]
         if len({w.dtype for w in weights}) != 1:
             raise TypeError("the projections of one layer must share a dtype to be stacked")
         keep = self.runtime.keep_plain_weights
         self.in_weight = Weight(torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0], keep_plain=keep)
         del weights
-        self.uq_weight = Weight(tensors[self.name("uq")], keep_plain=keep)
         self.o_weight = Weight(tensors[self.name("o")], keep_plain=keep)
-        self.q_norm = tensors[self.name("dq_norm")]
+        if self.q_rank:
+            self.uq_weight = Weight(tensors[self.name("uq")], keep_plain=keep)
+            self.q_norm = tensors[self.name("dq_norm")]
         if self.owns_kv:
             self.kv_norm = tensors[self.name("dkv_norm")]
         # per head [in, out]: Wuk_h as stored maps the latent to the head's dims, so read along its rows it folds a query
@@ -136,7 +145,8 @@ class LatentAttention(Mixer):
             stored = dict(pages=cache.rows, k_pages=None, v_pages=None, tiled_page_size=0)
         cq = kernels.latent_prepare(proj, self.q_at, self.q_rank, self.q_norm, self.kv_at, self.kv_rank, self.rot_dim, self.kv_norm,
                                     self.eps, cos_sin, view.slot_mapping if self.owns_kv else None, dtype, **stored)
-        q = linear(cq, self.uq_weight, out_dtype=torch.float32)         # rounded once, after folding and rotation
+        # the queries: through their latent, or columns of the stacked product; rounded once, after folding and rotation
+        q = linear(cq, self.uq_weight, out_dtype=torch.float32) if self.q_rank else proj[:, :self.q_width]
         q_full = torch.empty((n_tokens, self.heads * self.row), dtype=dtype, device=device)
         batched = dtype == torch.bfloat16 and n_tokens > self.BATCHED_ROWS
         if batched:
@@ -154,12 +164,13 @@ class LatentAttention(Mixer):
         else:
             weighted = kernels.latent_attention(q_full, cache.rows, view.block_table, ctx.seq_of_token, ctx.positions, self.scale,
                                                 self.window, self.heads, self.kv_rank, self.rot_dim)
-        gate = proj[:, self.gate_at:self.gate_at + self.heads * self.vdim] if self.output_gate else None
+        gate = proj[:, self.gate_at:self.gate_at + self.gate_width] if self.output_gate else None
         if batched:
-            o = kernels.gate_heads(torch.bmm(weighted.transpose(0, 1), self.unfold_values), gate)
+            o = kernels.gate_heads(torch.bmm(weighted.transpose(0, 1), self.unfold_values), gate, gate_a_head=self.gate_a_head)
         else:
             o = torch.empty((n_tokens, self.heads * self.vdim), dtype=dtype, device=device)
-            kernels.head_product(weighted, self.unfold_values, o.view(n_tokens, self.heads, self.vdim), gate=gate)
+            kernels.head_product(weighted, self.unfold_values, o.view(n_tokens, self.heads, self.vdim), gate=gate,
+                                 gate_a_head=self.gate_a_head)
         if residual is not None:
             begun = linear_into_stream(o, self.o_weight, residual)
             if begun is not None:

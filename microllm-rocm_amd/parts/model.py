@@ -54,6 +54,8 @@ class LMHead(Part):
         super().__init__(spec, runtime)
         self.vocab = int(spec.params["vocab_size"])
         self.width = int(spec.params["hidden_size"])
+        # ``softcap`` c: logits <- c * tanh(logits / c), in float32, after the product
+        self.softcap = float(spec.params["softcap"]) if spec.params.get("softcap") else 0.0
         self.weight: Optional[torch.Tensor] = None
 
     def tensors(self):
@@ -63,7 +65,8 @@ class LMHead(Part):
         self.weight = Weight(tensors[self.name("weight")], keep_plain=self.runtime.keep_plain_weights)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return linear(x, self.weight, out_dtype=torch.float32)
+        logits = linear(x, self.weight, out_dtype=torch.float32)
+        return kernels.softcap(logits, self.softcap) if self.softcap > 0.0 else logits
 
     def flops(self, tokens: int, wanted: int = 1) -> float:
         return 2.0 * self.vocab * self.width * wanted     # logits at the wanted rows only

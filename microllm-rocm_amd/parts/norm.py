@@ -16,6 +16,26 @@ from .registry import register_part
 from .spec import PartSpec
 
 
+class NormedDelta:
+    """A sublayer's result that is still to be RMS-normed with a weight of its own and multiplied by ``mult`` before
+    it joins the residual stream: ``h += mult * values / sqrt(mean(values^2) + eps) * weight``. The norm that reads the
+    stream next does both in one kernel. ``values`` is ``[tokens, hidden]`` or float32 partial sums ``[parts, tokens,
+    hidden]``, which are added in order first."""
+
+    def __init__(self, values: torch.Tensor, weight: torch.Tensor, eps: float, mult: float):
+        self.values = values
+        self.weight = weight
+        self.eps = float(eps)
+        self.mult = float(mult)
+
+    def resolved(self) -> torch.Tensor:
+        """What joins the stream, as a float32 tensor ``[tokens, hidden]`` (for observers; a step never needs it)."""
+        shape = self.values.shape[-2:]
+        joined = torch.zeros(shape, dtype=torch.float32, device=self.values.device)
+        kernels.rms_norm_after(joined, self.values, self.weight, self.eps, self.mult, None, 1.0, self.values.dtype, write_h=True)
+        return joined
+
+
 class RMSNorm(Norm):
     graph_safe = True
     def __init__(self, spec: PartSpec, runtime: Runtime):
@@ -39,6 +59,9 @@ class RMSNorm(Norm):
         return (self.weight, self.size, self.eps) if self.weight is not None and self.weight.dtype == torch.float32 else None
 
     def forward(self, h, delta=None, write_h=True, rows=None):
+        if isinstance(delta, NormedDelta):
+            return kernels.rms_norm_after(h, delta.values, delta.weight, delta.eps, delta.mult, self.weight, self.eps,
+                                          self.runtime.dtype, rows=rows, write_h=write_h and rows is None)
         return kernels.rms_norm(h, self.weight, self.eps, self.runtime.dtype, delta=delta, rows=rows,
                                 write_h=write_h and delta is not None and rows is None)
 

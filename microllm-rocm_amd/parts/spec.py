@@ -35,6 +35,7 @@ class LayerSpec:
     ffn_norm: Optional[PartSpec] = None
     ffn: Optional[PartSpec] = None
     extra: Mapping[str, Tuple[str, PartSpec]] = field(default_factory=dict)
+    params: Mapping[str, Any] = field(default_factory=dict)     # constants of the arrangement itself (a factor on what joins the stream)
 
 
 @dataclass(frozen=True)

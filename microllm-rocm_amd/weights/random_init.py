@@ -26,7 +26,7 @@ class InitRule:
     std_key: str
 
 
-DEFAULT_STDS = {"std": 0.02, "norm_std": 0.0, "connection_std": 0.0, "bias_std": 0.5}
+DEFAULT_STDS = {"std": 0.02, "norm_std": 0.0, "connection_std": 0.0, "bias_std": 0.5, "conv_std": 0.3}
 
 
 def _generator_for(seed: int, name: str, device: torch.device) -> torch.Generator:
