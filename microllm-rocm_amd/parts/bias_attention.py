@@ -84,7 +84,8 @@ class BucketBiasAttention(Mixer):
             raise ValueError("the keys and values must be kept at least as long as this layer's window")
         # the paged attention's pages and MFMA kernels, where they fit (the bias column must fit the prefill kernel's LDS;
         # slopes are such a column only under a window that fits)
-        table_rows = self.window if self.slope_values is not None else self.bias_max + 1
+        # (the widest window among the layers that share the pages decides, so that all of them lay the pages out alike)
+        table_rows = self.kept_window if self.slope_values is not None else self.bias_max + 1
         self.tiled = (bool(p.get("mfma", True)) and runtime.dtype == torch.bfloat16 and self.key_dim == self.value_dim
                       and self.key_dim % 16 == 0 and self.key_dim <= 256 and 0 < table_rows <= kernels.MFMA_BIAS_ROWS)
         self.planner = QueryTilePlanner(bool(self.window)) if self.tiled else None

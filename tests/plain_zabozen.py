@@ -91,20 +91,34 @@ def attention_keys_values(a: torch.Tensor, tensors, prefix: str, mixer: Mapping,
     return rms(k, eps), v
 
 
+def head_slopes(heads: int) -> List[float]:
+    return [2.0 ** (-8.0 * (h + 1) / heads) for h in range(heads)]
+
+
+def window_attention(q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float, window: int,
+                     slopes: Optional[List[float]]) -> torch.Tensor:
+    """``q [T, H, dim]``, ``keys [T, G, dim]``, ``values [T, G, vdim]`` -> ``[T, H, vdim]``: query ``i`` sees the keys
+    ``j`` with ``0 <= i - j < window`` (``window`` 0: all ``j <= i``); ``slopes[h] * (i - j)`` is taken off the score."""
+    T, H, G = q.shape[0], q.shape[1], keys.shape[1]
+    positions = torch.arange(T)
+    distance = positions[:, None] - positions[None, :]
+    visible = (distance >= 0) & ((distance < window) if window else (distance >= 0))
+    out = torch.zeros((T, H, values.shape[2]), dtype=F)
+    for h in range(H):
+        g = h // (H // G)
+        scores = (q[:, h] @ keys[:, g].T) * scale
+        if slopes is not None:
+            scores = scores - slopes[h] * distance.to(F)
+        out[:, h] = softmax_rows(scores, visible) @ values[:, g]
+    return out
+
+
 def attention(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps: float,
               keys: torch.Tensor, values: torch.Tensor) -> torch.Tensor:
     T = a.shape[0]
-    H, G, dim, vdim = mixer["heads"], mixer["kv_heads"], mixer["dim"], mixer["vdim"]
+    H, dim, vdim = mixer["heads"], mixer["dim"], mixer["vdim"]
     q = rms((a @ t64(tensors, f"{prefix}.q").T + t64(tensors, f"{prefix}.q.b")).view(T, H, dim), eps)
-    positions = torch.arange(T)
-    distance = positions[:, None] - positions[None, :]
-    visible = (distance >= 0) & (distance < mixer["mask"]["size"])
-    out = torch.zeros((T, H, vdim), dtype=F)
-    for h in range(H):
-        g = h // (H // G)
-        slope = 2.0 ** (-8.0 * (h + 1) / H)
-        scores = (q[:, h] @ keys[:, g].T) * mixer["scale"] - slope * distance.to(F)
-        out[:, h] = softmax_rows(scores, visible) @ values[:, g]
+    out = window_attention(q, keys, values, mixer["scale"], mixer["mask"]["size"], head_slopes(H))
     return out.reshape(T, H * vdim) @ t64(tensors, f"{prefix}.o").T + t64(tensors, f"{prefix}.o.b")
 
 
@@ -122,6 +136,26 @@ def unit(a: torch.Tensor) -> torch.Tensor:
     return a / torch.sqrt((a * a).sum(-1, keepdim=True) + 1e-6)
 
 
+def delta_walk(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor,
+               state: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``q, k [T, G, dim]``, ``v [T, H, vdim]``, ``beta, decay [T, H]``; ``state [H, dim, vdim]`` (zeros if None).
+    Returns the read-outs ``[T, H, vdim]`` and the state after the last token."""
+    T, G, dim = q.shape
+    H, vdim = v.shape[1], v.shape[2]
+    state = torch.zeros((H, dim, vdim), dtype=F) if state is None else state.clone()
+    out = torch.zeros((T, H, vdim), dtype=F)
+    for h in range(H):
+        g = h // (H // G)
+        S = state[h]
+        for t in range(T):
+            S = decay[t, h] * S
+            u = beta[t, h] * (v[t, h] - S.T @ k[t, g])
+            S = S + torch.outer(k[t, g], u)
+            out[t, h] = S.T @ q[t, g]
+        state[h] = S
+    return out, state
+
+
 def delta_rule(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps: float) -> torch.Tensor:
     T = a.shape[0]
     H, G, dim, vdim = mixer["heads"], mixer["kv_heads"], mixer["dim"], mixer["vdim"]
@@ -132,15 +166,7 @@ def delta_rule(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps: float
     beta = torch.sigmoid(a @ t64(tensors, f"{prefix}.b").T)                                     # [T, H]
     step = torch.nn.functional.softplus(a @ t64(tensors, f"{prefix}.a").T + t64(tensors, f"{prefix}.dt_bias"))
     decay = torch.exp(-torch.exp(t64(tensors, f"{prefix}.A_log")) * step)                       # [T, H]
-    out = torch.zeros((T, H, vdim), dtype=F)
-    for h in range(H):
-        g = h // (H // G)
-        S = torch.zeros((dim, vdim), dtype=F)
-        for t in range(T):
-            S = decay[t, h] * S
-            u = beta[t, h] * (v[t, h] - S.T @ k[t, g])
-            S = S + torch.outer(k[t, g], u)
-            out[t, h] = S.T @ q[t, g]
+    out, _ = delta_walk(q, k, v, beta, decay)
     gate = silu(a @ t64(tensors, f"{prefix}.g").T).view(T, H, vdim)
     out = rms(out, eps) * t64(tensors, f"{prefix}.norm") * gate
     return out.reshape(T, H * vdim) @ t64(tensors, f"{prefix}.o").T
@@ -183,3 +209,26 @@ def forward(config: Mapping, tensors: Mapping[str, torch.Tensor], tokens: List[i
     if cap:
         logits = cap * torch.tanh(logits / cap)
     return logits, torch.stack(streams)
+
+
+def read_config(folder: str) -> dict:
+    import json
+    import os
+    with open(os.path.join(folder, "config.json"), "r", encoding="utf-8") as handle:
+        return json.load(handle)
+
+
+def read_tensors(folder: str) -> Dict[str, torch.Tensor]:
+    import os
+    from safetensors.torch import load_file
+    return load_file(os.path.join(folder, "model.safetensors"))
+
+
+def generate_greedy(config: Mapping, tensors: Mapping[str, torch.Tensor], prompt: List[int], count: int) -> List[int]:
+    """``count`` tokens after ``prompt``, each the first maximum of the last position's logits; every step runs the
+    whole sequence again."""
+    tokens = list(prompt)
+    for _ in range(count):
+        logits, _ = forward(config, tensors, tokens)
+        tokens.append(int(torch.argmax(logits[-1])))
+    return tokens[len(prompt):]
