@@ -94,6 +94,29 @@ def gupitar_config(size: dict):
     return GupitarConfig(vocab=DESIGN_VOCAB, width=width, norm_eps=1e-6, layers=tuple(layers))
 
 
+def zabozen_config(size: dict):
+    """A Zabozen configuration of the given layer sizes: layers in turn a latent attention (heads of 96 unrotated and 64
+    rotated query/key dims and 128 value dims, cached rows of 192 + 64 elements, queries straight from the input, a
+    gate a head), a gated delta rule (as many value heads as the model has heads over its key/value head count of
+    key heads, 128 dims each, four taps), a window attention with slopes (the model's heads and key/value heads of the
+    head size, a window of 1024) and one on the keys and values of the layer before; every feed-forward dense."""
+    from microllm_rocm_amd.config.zabozen import (DeltaConfig, DenseMlpConfig, LatentAttentionConfig, WindowAttentionConfig,
+                                                  ZabozenConfig, ZabozenLayerConfig)
+    width, heads, kv_heads, dim = size["width"], size["heads"], size["kv_heads"], size["head_dim"]
+    layers = []
+    for index in range(size["layers"]):
+        kind = ("latent_attention", "delta", "attention", "borrow")[index % 4]
+        if kind == "latent_attention":
+            mixer = LatentAttentionConfig(heads=heads, dim=96, rot_dim=64, vdim=dim, kv_rank=192, scale=160 ** -0.5, rot_base=1e6, rot_dims=64)
+        elif kind == "delta":
+            mixer = DeltaConfig(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, conv=4)
+        else:
+            mixer = WindowAttentionConfig(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, window=1024,
+                                          kv_from=index - 1 if kind == "borrow" else None)
+        layers.append(ZabozenLayerConfig("attention" if kind == "borrow" else kind, mixer, DenseMlpConfig(size["ff"])))
+    return ZabozenConfig(vocab=DESIGN_VOCAB, width=width, norm_eps=1e-6, residual_mult=0.5, layers=tuple(layers), logit_softcap=30.0)
+
+
 def design_configs(size: dict, design: str = "siditar"):
     """The design's configuration at the given layer sizes and the Qwen2 configuration of equal width, heads, head size,
     feed-forward width, depth and vocabulary."""
@@ -104,6 +127,8 @@ def design_configs(size: dict, design: str = "siditar"):
                         tie_word_embeddings=False)
     if design == "gupitar":
         return {"gupitar": gupitar_config(size), "qwen2": qwen2}
+    if design == "zabozen":     # beside the design whose layers are most like its own, and beside Qwen2
+        return {"zabozen": zabozen_config(size), "gupitar": gupitar_config(size), "qwen2": qwen2}
     from microllm_rocm_amd.config.siditar import (BiasAttentionConfig, DenseMlpConfig, LinearAttentionConfig,
                                                   ParallelMixerConfig, SiditarConfig, SiditarLayerConfig)
     left = BiasAttentionConfig(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["head_dim"], vdim=size["head_dim"],
@@ -145,11 +170,12 @@ def compare_designs(args) -> int:
             del engine
             torch.cuda.empty_cache()
     first = next((row for row in rows if row["design"] == args.design), rows[0])
-    line = {"metric": f"decode tok/s of the {args.design.capitalize()} design beside Qwen2 at equal layer sizes", "value": first["decode"]["tok_per_s"],
+    others = " and ".join(name.capitalize() for name in design_configs(DESIGN_SIZES["1k"], args.design) if name != args.design)
+    line = {"metric": f"decode tok/s of the {args.design.capitalize()} design beside {others} at equal layer sizes", "value": first["decode"]["tok_per_s"],
             "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["decode"]["ms_per_step"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights, uniform-random token ids, caches filled with random keys and values",
-            "config": {"model": f"{args.design.capitalize()} and Qwen2 at sizes {args.design_sizes}", "global_batch": args.batch, "seq_len": args.context,
+            "config": {"model": f"{args.design.capitalize()} and {others} at sizes {args.design_sizes}", "global_batch": args.batch, "seq_len": args.context,
                        "vocab": DESIGN_VOCAB, "kv_block_size": page_size, "parallelism": "single GPU"},
             "compare": rows}
     print(json.dumps(line), flush=True)
@@ -182,11 +208,11 @@ def main() -> int:
     parser.add_argument("--no-extras", action="store_true",
                         help="leave out what the default run adds to its line after the main figures: decoding on the 32-bit path "
                              "at batch 8 and the continuous-batching workload at Qwen2-0.5B sizes")
-    parser.add_argument("--design", default=None, choices=["siditar", "gupitar"],
+    parser.add_argument("--design", default=None, choices=["siditar", "gupitar", "zabozen"],
                         help="instead of the default workload: prefill and decode throughput of this design beside Qwen2 at equal "
                              "layer sizes (--design-sizes), random weights; --batch, --context, --prefill-tokens, --steps apply")
     parser.add_argument("--design-sizes", default="1k,2k,4k", help="of " + ", ".join(sorted(DESIGN_SIZES)))
-    parser.add_argument("--design-only", default=None, choices=["siditar", "gupitar", "qwen2"], help="one of the two designs alone (profiles)")
+    parser.add_argument("--design-only", default=None, choices=["siditar", "gupitar", "zabozen", "qwen2"], help="one of the designs alone (profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
