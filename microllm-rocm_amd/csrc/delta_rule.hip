@@ -190,6 +190,182 @@ delta_scan_kernel(const float* __restrict__ u, const float* __restrict__ gates, 
     }
 }
 
+
+// The same walk for portions of many tokens: a wave brings tiles of tokens (keys and queries of its key head, the
+// values of its columns, the head's two gates) from memory straight into LDS, the next tile on its way while it
+// walks this one, so that a token waits for LDS and not for memory. The operations per token and their order are
+// those of the kernel above: the same bits, only where the operands come from differs.
+// WIDE: rows of key channels and their places in memory are multiples of 16 bytes, and a lane's load brings 16.
+constexpr int kDeltaTileFloats = 2048;      // of each of keys and queries in a tile
+constexpr int kDeltaTileTokens = 64;        // at most
+constexpr int kDeltaBufferFloats = 2 * kDeltaTileFloats + kDeltaTileTokens * (kDeltaColumnsAWave + 2);
+
+template <bool WIDE, int ROWS>
+__global__ void __launch_bounds__(kWave)
+delta_scan_tiled_kernel(const float* __restrict__ u, const float* __restrict__ gates, float* __restrict__ state,
+                        const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ slots, float* __restrict__ out,
+                        int key_heads, int heads, int key_dim, int value_dim) {
+    __shared__ __align__(16) float buffer_even[kDeltaBufferFloats];
+    __shared__ __align__(16) float buffer_odd[kDeltaBufferFloats];
+    constexpr int kRowFloats = ROWS * kDeltaLanesAColumn;                                      // a token's row of key channels in LDS
+    constexpr int kTileTokens = kDeltaTileFloats / kRowFloats < kDeltaTileTokens ? kDeltaTileFloats / kRowFloats : kDeltaTileTokens;
+    constexpr int kValuesAt = 2 * kDeltaTileFloats, kGatesAt = kValuesAt + kDeltaTileTokens * kDeltaColumnsAWave;
+    const int seq = blockIdx.x;
+    const int head = blockIdx.y;
+    const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+    if (last <= first) return;
+    const int lane = threadIdx.x;
+    const int r = lane % kDeltaLanesAColumn;
+    const int column_in_wave = lane / kDeltaLanesAColumn;
+    const int column = blockIdx.z * kDeltaColumnsAWave + column_in_wave;
+    const bool live = column < value_dim;
+    const int safe_column = live ? column : 0;
+    const int key_head = head / (heads / key_heads);
+    const int channels = 2 * key_heads * key_dim + heads * value_dim;
+    const int q_at = key_head * key_dim, k_at = (key_heads + key_head) * key_dim;
+    const int v_at = 2 * key_heads * key_dim + head * value_dim;
+    float* mine = state + ((static_cast<int64_t>(slots[seq]) * heads + head) * key_dim) * value_dim + safe_column;
+    float s[ROWS];
+    bool valid[ROWS];
+    bool all_valid = true;
+#pragma unroll
+    for (int m = 0; m < ROWS; ++m) {
+        const int i = ROWS * r + m;
+        valid[m] = i < key_dim;
+        all_valid = all_valid && valid[m];
+        s[m] = valid[m] ? mine[static_cast<int64_t>(i) * value_dim] : 0.0f;
+    }
+    all_valid = __all(all_valid);
+    // Nothing that is read from LDS may be a stray bit pattern: places that no load fills are read beside others.
+    for (int index = lane; index < kDeltaBufferFloats; index += kWave) buffer_even[index] = buffer_odd[index] = 0.0f;
+    __syncthreads();
+    // Which token of a tile and which channel each of this lane's loads brings (the same for every tile). A row's
+    // places beyond key_dim bring a channel of the row again; the walk never lets them count.
+    constexpr int kPiece = WIDE ? 4 : 1;                                        // floats a lane's load brings
+    constexpr int kCalls = kTileTokens * kRowFloats / (kWave * kPiece);         // loads that bring one of keys, queries
+    int token_of[kCalls], channel_of[kCalls];
+#pragma unroll
+    for (int j = 0; j < kCalls; ++j) {
+        const int element = (j * kWave + lane) * kPiece;
+        token_of[j] = element / kRowFloats;
+        channel_of[j] = min(element % kRowFloats, key_dim - kPiece);
+    }
+    constexpr int kValueCalls = (kTileTokens * kDeltaColumnsAWave + kWave - 1) / kWave;
+    constexpr int kGateCalls = (kTileTokens * 2 + kWave - 1) / kWave;
+    auto fetch = [&](int tile_first, float* buffer) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < kCalls; ++j) {
+            const int64_t token = min(tile_first + token_of[j], last - 1);
+            const float* row = u + token * channels + channel_of[j];
+            float* place = buffer + j * kWave * kPiece;
+            if constexpr (WIDE) {
+                __builtin_amdgcn_global_load_lds(row + k_at, place, 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(row + q_at, place + kDeltaTileFloats, 16, 0, 0);
+            } else {
+                __builtin_amdgcn_global_load_lds(row + k_at, place, 4, 0, 0);
+                __builtin_amdgcn_global_load_lds(row + q_at, place + kDeltaTileFloats, 4, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kValueCalls; ++j) {
+            const int element = j * kWave + lane;
+            const int64_t token = min(tile_first + element / kDeltaColumnsAWave, last - 1);
+            const int wanted = min(static_cast<int>(blockIdx.z) * kDeltaColumnsAWave + element % kDeltaColumnsAWave, value_dim - 1);
+            __builtin_amdgcn_global_load_lds(u + token * channels + v_at + wanted, buffer + kValuesAt + j * kWave, 4, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < kGateCalls; ++j) {
+            const int element = j * kWave + lane;
+            const int64_t token = min(tile_first + element / 2, last - 1);
+            __builtin_amdgcn_global_load_lds(gates + token * 2 * heads + 2 * head + element % 2, buffer + kGatesAt + j * kWave, 4, 0, 0);
+        }
+    };
+    auto walk_tokens = [&](auto every_channel, int tile_first, int count, const float* buffer) __attribute__((always_inline)) {
+        // Two sets of a token's operands take turns: while one token is worked, the next one's leave LDS.
+        float k_a[ROWS], q_a[ROWS], k_b[ROWS], q_b[ROWS];
+        float few_a[3], few_b[3];       // value, beta, g
+        auto read_token = [&](int t, float* k, float* q, float* few) __attribute__((always_inline)) {
+            const float* row = buffer + t * kRowFloats + ROWS * r;
+            if constexpr (ROWS % 4 == 0) {
+#pragma unroll
+                for (int piece = 0; piece < ROWS; piece += 4) {
+                    *reinterpret_cast<float4*>(k + piece) = *reinterpret_cast<const float4*>(row + piece);
+                    *reinterpret_cast<float4*>(q + piece) = *reinterpret_cast<const float4*>(row + kDeltaTileFloats + piece);
+                }
+            } else {
+#pragma unroll
+                for (int m = 0; m < ROWS; ++m) k[m] = row[m], q[m] = row[kDeltaTileFloats + m];
+            }
+            if constexpr (!decltype(every_channel)::value) {
+#pragma unroll
+                for (int m = 0; m < ROWS; ++m) {
+                    k[m] = valid[m] ? k[m] : 0.0f;
+                    q[m] = valid[m] ? q[m] : 0.0f;
+                }
+            }
+            few[0] = buffer[kValuesAt + t * kDeltaColumnsAWave + column_in_wave];
+            few[1] = buffer[kGatesAt + 2 * t];
+            few[2] = buffer[kGatesAt + 2 * t + 1];
+        };
+        float* to = out + (static_cast<int64_t>(tile_first) * heads + head) * value_dim + column;
+        const int64_t to_stride = static_cast<int64_t>(heads) * value_dim;
+        const bool writes = live && r == 0;
+        auto work = [&](const float* k, const float* q, const float* few) __attribute__((always_inline)) {
+            const float v = few[0], beta = few[1], g = few[2];
+            float seen = 0.0f;
+#pragma unroll
+            for (int m = 0; m < ROWS; ++m) {
+                s[m] *= g;
+                seen = fmaf(s[m], k[m], seen);
+            }
+            const float correction = beta * (v - sum_row_of_16(seen));
+            float read = 0.0f;
+#pragma unroll
+            for (int m = 0; m < ROWS; ++m) {
+                s[m] = fmaf(k[m], correction, s[m]);
+                read = fmaf(s[m], q[m], read);
+            }
+            read = sum_row_of_16(read);
+            if (writes) *to = read;
+            to += to_stride;
+        };
+        read_token(0, k_a, q_a, few_a);
+        int t = 0;
+        for (; t + 1 < count; t += 2) {
+            read_token(t + 1, k_b, q_b, few_b);
+            work(k_a, q_a, few_a);
+            read_token(min(t + 2, count - 1), k_a, q_a, few_a);
+            work(k_b, q_b, few_b);
+        }
+        if (t < count) work(k_a, q_a, few_a);
+    };
+    auto walk = [&](int tile_first, const float* buffer) __attribute__((always_inline)) {
+        const int count = min(kTileTokens, last - tile_first);
+        if (all_valid) walk_tokens(std::true_type{}, tile_first, count, buffer);
+        else walk_tokens(std::false_type{}, tile_first, count, buffer);
+    };
+    fetch(first, buffer_even);
+    for (int tile_first = first; tile_first < last;) {
+        wait_for_loads();
+        __syncthreads();
+        if (tile_first + kTileTokens < last) fetch(tile_first + kTileTokens, buffer_odd);
+        walk(tile_first, buffer_even);
+        tile_first += kTileTokens;
+        if (tile_first >= last) break;
+        wait_for_loads();
+        __syncthreads();
+        if (tile_first + kTileTokens < last) fetch(tile_first + kTileTokens, buffer_even);
+        walk(tile_first, buffer_odd);
+        tile_first += kTileTokens;
+    }
+    if (!live) return;
+#pragma unroll
+    for (int m = 0; m < ROWS; ++m) {
+        const int i = ROWS * r + m;
+        if (i < key_dim) mine[static_cast<int64_t>(i) * value_dim] = s[m];
+    }
+}
+
 }  // namespace mll
 
 using namespace mll;
@@ -226,7 +402,7 @@ int mll_conv_keep(const float* proj, int64_t proj_stride, int conv_at, float* ke
 }
 
 int mll_delta_scan(const float* u, const float* gates, float* state, const int32_t* cu_tokens, const int32_t* slots, float* out,
-                   int n_seqs, int key_heads, int heads, int key_dim, int value_dim, hipStream_t stream) {
+                   int n_seqs, int key_heads, int heads, int key_dim, int value_dim, int long_portions, hipStream_t stream) {
     MLL_REQUIRE(n_seqs >= 0 && key_heads > 0 && heads > 0 && key_dim > 0 && value_dim > 0, "delta_scan: sizes must be positive");
     MLL_REQUIRE(heads % key_heads == 0, "delta_scan: the value heads must divide into the key heads");
     MLL_REQUIRE(key_dim <= 16 * kDeltaLanesAColumn, "delta_scan: key heads wider than 256 are not supported");
@@ -235,6 +411,22 @@ int mll_delta_scan(const float* u, const float* gates, float* state, const int32
     MLL_REQUIRE(heads < 65536 && groups < 65536, "delta_scan: too many heads or value channels for one launch");
     const dim3 grid(n_seqs, heads, groups);
     const int rows = (key_dim + kDeltaLanesAColumn - 1) / kDeltaLanesAColumn;
+    if (long_portions) {
+        const int channels = 2 * key_heads * key_dim + heads * value_dim;
+        const bool wide = key_dim % 4 == 0 && channels % 4 == 0 && reinterpret_cast<uintptr_t>(u) % 16 == 0;
+#define MLL_DELTA_TILED(WIDE, ROWS) \
+    delta_scan_tiled_kernel<WIDE, ROWS><<<grid, kWave, 0, stream>>>(u, gates, state, cu_tokens, slots, out, key_heads, heads, key_dim, value_dim)
+#define MLL_DELTA_TILED_ROWS(ROWS) \
+    do { if (wide) MLL_DELTA_TILED(true, ROWS); else MLL_DELTA_TILED(false, ROWS); } while (0)
+        if (rows <= 1) MLL_DELTA_TILED(false, 1);
+        else if (rows <= 2) MLL_DELTA_TILED(false, 2);
+        else if (rows <= 4) MLL_DELTA_TILED_ROWS(4);
+        else if (rows <= 8) MLL_DELTA_TILED_ROWS(8);
+        else MLL_DELTA_TILED_ROWS(16);
+#undef MLL_DELTA_TILED_ROWS
+#undef MLL_DELTA_TILED
+        return check_launch("delta_scan_tiled");
+    }
 #define MLL_DELTA_SCAN(ROWS) \
     delta_scan_kernel<ROWS><<<grid, kWave, 0, stream>>>(u, gates, state, cu_tokens, slots, out, key_heads, heads, key_dim, value_dim)
     if (rows <= 1) MLL_DELTA_SCAN(1);

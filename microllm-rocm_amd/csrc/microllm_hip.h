@@ -386,8 +386,10 @@ int mll_conv_keep(const float* proj, int64_t proj_stride, int conv_at, float* ke
 
 // Per request and head, over the request's tokens in order, with S = state[slot][head] ([key_dim][value_dim], read
 // first, written last): S *= g; c = beta * (v - S^T k); S += k c^T; out[t][head] = S^T q. u and gates as above.
+// long_portions: the kernel that stages tiles of tokens through LDS, for steps whose requests bring many tokens (the
+// same bits).
 int mll_delta_scan(const float* u, const float* gates, float* state, const int32_t* cu_tokens, const int32_t* slots, float* out,
-                   int n_seqs, int key_heads, int heads, int key_dim, int value_dim, hipStream_t stream);
+                   int n_seqs, int key_heads, int heads, int key_dim, int value_dim, int long_portions, hipStream_t stream);
 
 // ---- a recurrent block with a gated linear recurrence (csrc/recurrent.hip) ----------------------------------------
 

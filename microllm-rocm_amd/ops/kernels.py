@@ -1409,10 +1409,12 @@ def conv_keep(proj: torch.Tensor, conv_at: int, kept: torch.Tensor, cu_tokens: t
 
 
 def delta_scan(u: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, cu_tokens: torch.Tensor, slots: torch.Tensor,
-               n_seqs: int, key_heads: int, heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
+               n_seqs: int, key_heads: int, heads: int, key_dim: int, value_dim: int, long_portions: bool = False) -> torch.Tensor:
     """The delta rule over every request's tokens of the step, in order: ``S *= g; c = beta (v - S^T k); S += k c^T;
     o = S^T q`` with ``S = state[slot, head]`` (``[slots, heads, key_dim, value_dim]`` float32, read first and written
-    last). ``u`` and ``gates`` as ``delta_prepare`` returns them. Returns ``[tokens, heads * value_dim]`` float32."""
+    last). ``u`` and ``gates`` as ``delta_prepare`` returns them. Returns ``[tokens, heads * value_dim]`` float32.
+    ``long_portions``: the kernel that stages tiles of tokens through LDS, for steps whose requests bring many tokens
+    (the same bits)."""
     lib = library.load()
     _device_tensor(u, "queries, keys and values", torch.float32)
     _device_tensor(gates, "gates", torch.float32)
@@ -1425,8 +1427,9 @@ def delta_scan(u: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, cu_tok
     _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, key_dim, value_dim), "state is [slots, heads, key_dim, value_dim]")
     _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
     out = torch.empty((n_tokens, heads * value_dim), dtype=torch.float32, device=u.device)
+    _need(u.is_contiguous() and gates.is_contiguous(), "u and gates are contiguous")
     _check(lib.mll_delta_scan(_ptr(u), _ptr(gates), _ptr(state), _ptr(cu_tokens), _ptr(slots), _ptr(out), n_seqs, key_heads, heads,
-                              key_dim, value_dim, _stream()), lib)
+                              key_dim, value_dim, int(long_portions), _stream()), lib)
     return out
 
 

@@ -33,6 +33,7 @@ class GatedDeltaRule(Mixer):
     # A step that is run twice would change the state twice: the engine, which runs a step once before it captures
     # it, saves the step's state slots before that run and puts them back.
     graph_safe = True
+    LONG_PORTION = 8        # from this many tokens of one request in a step on, the walk stages its operands through LDS
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
@@ -94,7 +95,7 @@ class GatedDeltaRule(Mixer):
         if self.taps > 1:
             kernels.conv_keep(proj, self.conv_at, kept, ctx.cu_tokens, ctx.slots, ctx.n_seqs)
         o = kernels.delta_scan(u, gates, state, ctx.cu_tokens, ctx.slots, ctx.n_seqs, self.key_heads, self.heads, self.key_dim,
-                               self.value_dim)
+                               self.value_dim, long_portions=ctx.max_count >= self.LONG_PORTION)
         gated = kernels.gla_gate(o, proj, self.gate_at, self.norm_weight, self.eps, self.heads, self.value_dim, 1.0, self.runtime.dtype)
         return linear(gated, self.o_weight, out_dtype=torch.float32, partials=True)
 

@@ -156,7 +156,8 @@ def plain_delta(proj, taps, a_log, dt_bias, key_heads, heads, key_dim, value_dim
 
 
 @pytest.mark.parametrize("key_heads,heads,key_dim,value_dim,taps", [(2, 6, 12, 10, 3), (1, 1, 9, 14, 1), (3, 3, 40, 7, 2), (1, 4, 128, 24, 5),
-                                                                    (2, 2, 200, 5, 4), (1, 2, 16, 64, 4)])
+                                                                    (2, 2, 200, 5, 4), (1, 2, 16, 64, 4), (2, 2, 26, 3, 2), (1, 3, 64, 8, 3),
+                                                                    (1, 1, 256, 4, 2), (1, 2, 100, 9, 4)])
 def test_delta_rule_in_steps_with_carried_state(key_heads, heads, key_dim, value_dim, taps):
     """Convolution, unit vectors, gates, the walk, the norm and gate of the result: two requests in one step, then
     continued one and two tokens at a time beside a third that starts, in slots that are not in order and hold what
@@ -191,7 +192,10 @@ def test_delta_rule_in_steps_with_carried_state(key_heads, heads, key_dim, value
                                          key_dim ** -0.5, 1e-6)
         if taps > 1:
             kernels.conv_keep(proj, 0, kept, cu, slots, len(names))
+        state_before = state.clone()      # the walk that stages tiles of tokens through LDS leaves the same bits
+        staged = kernels.delta_scan(u, gates, state_before, cu, slots, len(names), key_heads, heads, key_dim, value_dim, long_portions=True)
         o = kernels.delta_scan(u, gates, state, cu, slots, len(names), key_heads, heads, key_dim, value_dim)
+        assert torch.equal(staged, o) and torch.equal(state_before, state)
         out = kernels.gla_gate(o, proj, channels, device(norm_weight), 1e-5, heads, value_dim, 1.0, torch.float32).cpu().numpy()
         first = 0
         for name in names:
