@@ -8,7 +8,9 @@
 // by a factor; beta = sigmoid(.) and g = exp(-exp(A_log) * softplus(. + dt_bias)) are one number a head and token.
 // Three kernels: the convolution with its activation, the unit vectors and the two gates for all tokens of a step at
 // once; the newest inputs of the convolution into the request's slot; and the walk over each request's tokens in
-// order. The columns of S are independent, so a head is spread over waves by value channel. Everything is float32.
+// order (in two forms: operands straight from memory for steps of few tokens a request, tiles of tokens staged through
+// LDS for portions of prompts). The columns of S are independent, so a head is spread over waves by value channel.
+// Everything is float32.
 #include "common.h"
 #include "microllm_hip.h"
 

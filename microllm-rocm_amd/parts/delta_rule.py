@@ -14,7 +14,10 @@ so the read-out sees the token's own write. Each head's ``o`` is divided by its 
 multiplied by a weight ``[value_dim]`` that all heads share and by ``silu(Wg x)``, and projected by ``Wo``. A request
 keeps ``S`` and the convolution's last ``taps - 1`` inputs, both float32, in its state slot, so it can be cut into steps
 anywhere. The six projections that read ``x`` are one stacked product with a float32 result; the convolution, the unit
-vectors, the gates, the recurrence, the norm and the output gate are float32.
+vectors, the gates, the recurrence, the norm and the output gate are float32. Steps in which a request brings
+``LONG_PORTION`` tokens or more walk the recurrence on the kernel that stages tiles of tokens through LDS; it does the
+same operations in the same order as the one that reads a token's operands from memory, so the state's bits do not
+depend on how a request was cut.
 """
 from __future__ import annotations
 
