@@ -1,2 +1,2 @@
 """Architectures this package provides; importing the package registers them."""
-from . import gupitar, qwen2, siditar, zabozen  # noqa: F401
+from . import gupitar, kalevik, qwen2, siditar, zabozen  # noqa: F401

@@ -66,7 +66,8 @@ bias_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
                       const int32_t* __restrict__ positions, const float* __restrict__ bias, int longest,
                       const float* __restrict__ sink, T* __restrict__ out, int64_t out_stride, int heads, int kv_heads,
                       int key_dim, int value_dim, int page_size, float scale, float out_scale,
-                      const float* __restrict__ slopes, int window) {
+                      const float* __restrict__ slopes, int window, int chunk, const float* __restrict__ gate,
+                      int64_t gate_stride) {
     extern __shared__ float q_row[];
     const int token = blockIdx.x / heads;
     const int head = blockIdx.x % heads;
@@ -85,7 +86,8 @@ bias_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
     const int64_t key_row = static_cast<int64_t>(kv_heads) * key_dim;
     const int64_t value_row = static_cast<int64_t>(kv_heads) * value_dim;
     const float slope = slopes ? slopes[head] : 0.0f;
-    const int low = window > 0 ? max(0, position - window + 1) : 0;     // the oldest key seen
+    // the oldest key seen: the first of the query's chunk of positions, or what the window reaches back to
+    const int low = chunk > 0 ? position / chunk * chunk : (window > 0 ? max(0, position - window + 1) : 0);
     for (int first = low / kBiasKeyTile * kBiasKeyTile; first <= position; first += kBiasKeyTile) {
         const int j = first + lane;
         float score = -INFINITY;
@@ -118,7 +120,8 @@ bias_attention_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
             }
         }
     }
-    const float factor = out_scale / running_sum;
+    float factor = out_scale / running_sum;
+    if (gate) factor *= 1.0f / (1.0f + expf(-gate[static_cast<int64_t>(token) * gate_stride + head]));
     T* to = out + static_cast<int64_t>(token) * out_stride + static_cast<int64_t>(head) * value_dim;
 #pragma unroll
     for (int m = 0; m < kMaxValueChannelsALane; ++m) {
@@ -135,13 +138,13 @@ qk_norm_store_kernel(const float* __restrict__ qkv, int n_parts, int64_t part_st
                      const float* __restrict__ k_weight, float eps, const int32_t* __restrict__ positions,
                      const int32_t* __restrict__ slot_mapping, float temp_coef, int temp_every, T* __restrict__ q_out,
                      T* __restrict__ k_pages, T* __restrict__ v_pages, int heads, int kv_heads, int key_dim, int value_dim,
-                     int tiled_page_size, const float* __restrict__ bias, int normed, int queries_only) {
+                     int tiled_page_size, const float* __restrict__ bias, int normed, int queries_only, int64_t row_stride,
+                     const float* __restrict__ cos_sin, int rot_dims) {
     const int vectors = queries_only ? heads : heads + 2 * kv_heads;
     const int token = blockIdx.x / vectors;
     const int which = blockIdx.x % vectors;
     const int lane = threadIdx.x;
-    const int row_width = queries_only ? heads * key_dim : (heads + kv_heads) * key_dim + kv_heads * value_dim;
-    const float* row = qkv + static_cast<int64_t>(token) * row_width;
+    const float* row = qkv + static_cast<int64_t>(token) * row_stride;
     const bool is_q = which < heads, is_k = !is_q && which < heads + kv_heads;
     const int head = is_q ? which : (is_k ? which - heads : which - heads - kv_heads);
     const int dim = (is_q || is_k) ? key_dim : value_dim;
@@ -171,11 +174,26 @@ qk_norm_store_kernel(const float* __restrict__ qkv, int n_parts, int64_t part_st
     const CacheLayout layout(kv_heads, tiled ? tiled_page_size : 16, key_dim);
     const int64_t page = tiled ? slot / tiled_page_size : 0;
     const int in_page = tiled ? slot % tiled_page_size : 0;
-    for (int c = lane; c < dim; c += kWave) {
+    // what the vector holds at channel c before it is turned: the sums, the bias, the norm
+    auto prepared = [&](int c) {
         float value = row[offset + c];
         for (int part = 1; part < n_parts; ++part) value += row[part * part_stride + offset + c];
         if (bias) value += bias[offset + c];
-        const T rounded = from_float<T>(norm ? (weight ? value * factor * weight[c] : value * factor) : value);
+        return norm ? (weight ? value * factor * weight[c] : value * factor) : value;
+    };
+    // queries and keys turn by the token's position in their first rot_dims channels, channel i with i + rot_dims / 2
+    const bool turns = cos_sin != nullptr && (is_q || is_k);
+    const int half = rot_dims / 2;
+    const float* angles = cos_sin + static_cast<int64_t>(token) * rot_dims;     // [rot_dims / 2][cos, sin]
+    for (int c = lane; c < dim; c += kWave) {
+        float value = prepared(c);
+        if (turns && c < rot_dims) {
+            const int pair = c < half ? c : c - half;
+            const float other = prepared(c < half ? c + half : c - half);
+            const float cosine = angles[2 * pair], sine = angles[2 * pair + 1];
+            value = c < half ? value * cosine - other * sine : value * cosine + other * sine;
+        }
+        const T rounded = from_float<T>(value);
         if (tiled) {
             if (is_k) k_pages[layout.k_at(page, head, in_page, c)] = rounded;
             else v_pages[layout.v_at(page, head, in_page, c)] = rounded;
@@ -194,11 +212,16 @@ extern "C" {
 int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const float* q_weight, const float* k_weight,
                       float eps, const int32_t* positions, const int32_t* slot_mapping, float temp_coef, int temp_every,
                       void* q_out, void* k_pages, void* v_pages, int dtype, int n_tokens, int heads, int kv_heads, int key_dim,
-                      int value_dim, int tiled_page_size, const float* bias, int normed, int queries_only, hipStream_t stream) {
+                      int value_dim, int tiled_page_size, const float* bias, int normed, int queries_only, int64_t row_stride,
+                      const float* cos_sin, int rot_dims, hipStream_t stream) {
     MLL_REQUIRE(tiled_page_size == 0 || (tiled_page_size > 0 && tiled_page_size % 16 == 0 && key_dim == value_dim),
                 "qk_norm_store: tiled pages hold a multiple of 16 positions and keys and values of one width");
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0, "qk_norm_store: sizes must be positive");
     MLL_REQUIRE(n_parts >= 1, "qk_norm_store: at least one part");
+    MLL_REQUIRE(row_stride >= (queries_only ? heads * key_dim : (heads + kv_heads) * key_dim + kv_heads * value_dim),
+                "qk_norm_store: the rows are narrower than their queries, keys and values");
+    MLL_REQUIRE(cos_sin == nullptr || (rot_dims > 0 && rot_dims % 2 == 0 && rot_dims <= key_dim),
+                "qk_norm_store: an even number of turned channels, at most the head's");
     MLL_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qk_norm_store: norm weights for queries and keys, or for neither");
     MLL_REQUIRE(!normed || eps > 0.0f, "qk_norm_store: eps must be positive");
     MLL_REQUIRE(normed || q_weight == nullptr, "qk_norm_store: norm weights without a norm");
@@ -211,12 +234,12 @@ int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const 
         qk_norm_store_kernel<float><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
             qkv, n_parts, part_stride, q_weight, k_weight, eps, positions, slot_mapping, temp_coef, temp_every,
             static_cast<float*>(q_out), static_cast<float*>(k_pages), static_cast<float*>(v_pages), heads, kv_heads, key_dim, value_dim,
-            tiled_page_size, bias, normed, queries_only);
+            tiled_page_size, bias, normed, queries_only, row_stride, cos_sin, rot_dims);
     } else if (dtype == kBF16) {
         qk_norm_store_kernel<bf16><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
             qkv, n_parts, part_stride, q_weight, k_weight, eps, positions, slot_mapping, temp_coef, temp_every,
             static_cast<bf16*>(q_out), static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), heads, kv_heads, key_dim, value_dim,
-            tiled_page_size, bias, normed, queries_only);
+            tiled_page_size, bias, normed, queries_only, row_stride, cos_sin, rot_dims);
     } else {
         return fail("qk_norm_store: unknown dtype");
     }
@@ -227,13 +250,15 @@ int mll_bias_attention(const void* q, const void* k_pages, const void* v_pages, 
                        const int32_t* seq_of_token, const int32_t* positions, const float* bias, int longest,
                        const float* sink, void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int kv_heads,
                        int key_dim, int value_dim, int page_size, float scale, float out_scale, const float* slopes, int window,
-                       hipStream_t stream) {
+                       int chunk, const float* gate, int64_t gate_stride, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0 && page_size > 0 && table_width > 0,
                 "bias_attention: sizes must be positive");
     MLL_REQUIRE(heads % kv_heads == 0, "bias_attention: heads must divide into kv heads");
     MLL_REQUIRE(value_dim <= kMaxValueChannelsALane * kWave, "bias_attention: value heads wider than 256 are not supported");
     MLL_REQUIRE(bias == nullptr || longest >= 0, "bias_attention: the bias table needs at least one row");
     MLL_REQUIRE(out_stride >= static_cast<int64_t>(heads) * value_dim, "bias_attention: the output rows overlap");
+    MLL_REQUIRE(window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0), "bias_attention: a window or chunks of positions, not both");
+    MLL_REQUIRE(gate == nullptr || gate_stride >= heads, "bias_attention: one gate a head in every row");
     if (n_tokens == 0) return 0;
     const int64_t blocks = static_cast<int64_t>(n_tokens) * heads;
     MLL_REQUIRE(blocks < (1ll << 31), "bias_attention: too many rows for one launch");
@@ -243,12 +268,12 @@ int mll_bias_attention(const void* q, const void* k_pages, const void* v_pages, 
         bias_attention_kernel<float><<<static_cast<unsigned>(blocks), kWave, lds, stream>>>(
             static_cast<const float*>(q), static_cast<const float*>(k_pages), static_cast<const float*>(v_pages), block_table,
             table_width, seq_of_token, positions, bias, longest, sink, static_cast<float*>(out), out_stride, heads, kv_heads,
-            key_dim, value_dim, page_size, scale, out_scale, slopes, window);
+            key_dim, value_dim, page_size, scale, out_scale, slopes, window, chunk, gate, gate_stride);
     } else if (dtype == kBF16) {
         bias_attention_kernel<bf16><<<static_cast<unsigned>(blocks), kWave, lds, stream>>>(
             static_cast<const bf16*>(q), static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages), block_table,
             table_width, seq_of_token, positions, bias, longest, sink, static_cast<bf16*>(out), out_stride, heads, kv_heads,
-            key_dim, value_dim, page_size, scale, out_scale, slopes, window);
+            key_dim, value_dim, page_size, scale, out_scale, slopes, window, chunk, gate, gate_stride);
     } else {
         return fail("bias_attention: unknown dtype");
     }

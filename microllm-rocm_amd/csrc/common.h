@@ -79,6 +79,14 @@ template <> __host__ __device__ inline bf16 from_float<bf16>(float value) {
     return out;
 }
 
+// The activations a kernel may be asked for by number: 0 SiLU, 1 the exact gelu, 2 the tanh form of gelu.
+constexpr int kActSilu = 0, kActGeluErf = 1, kActGeluTanh = 2;
+__device__ inline float activate(float z, int act) {
+    if (act == kActGeluErf) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));
+    if (act == kActGeluTanh) return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+    return z / (1.0f + expf(-z));
+}
+
 __device__ inline float wave_sum(float value) {
 #pragma unroll
     for (int offset = kWave / 2; offset > 0; offset >>= 1) value += __shfl_xor(value, offset, kWave);

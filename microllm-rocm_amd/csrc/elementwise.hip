@@ -16,7 +16,7 @@ int fail(const std::string& text) {
 // ---------------------------------------------------------------------------------------------
 template <typename W>
 __global__ void embedding_kernel(const W* __restrict__ table, const int32_t* __restrict__ ids,
-                                 float* __restrict__ out, int width, int vocab) {
+                                 float* __restrict__ out, int width, int vocab, float scale) {
     const int token = blockIdx.x;
     const int id = ids[token];
     float* row_out = out + static_cast<int64_t>(token) * width;
@@ -25,7 +25,7 @@ __global__ void embedding_kernel(const W* __restrict__ table, const int32_t* __r
         return;
     }
     const W* row = table + static_cast<int64_t>(id) * width;
-    for (int column = threadIdx.x; column < width; column += blockDim.x) row_out[column] = to_float(row[column]);
+    for (int column = threadIdx.x; column < width; column += blockDim.x) row_out[column] = to_float(row[column]) * scale;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -415,6 +415,19 @@ __global__ void silu_mul_bf16x8_kernel(const bf16* __restrict__ gate, const bf16
     *reinterpret_cast<uint4*>(out + static_cast<int64_t>(token) * width + chunk * 8) = z.raw;
 }
 
+
+// out[i] = act(in[i]): in float32 (partial sums added in order first) or T; act 0 SiLU, 1 the exact gelu
+// 0.5 z (1 + erf(z / sqrt 2)), 2 the tanh form of gelu.
+template <typename T, typename S>
+__global__ void __launch_bounds__(256)
+activation_kernel(const S* __restrict__ in, int n_parts, int64_t part_stride, T* __restrict__ out, int64_t count, int act) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float z = to_float(in[i]);
+    for (int part = 1; part < n_parts; ++part) z += to_float(in[part * part_stride + i]);
+    out[i] = from_float<T>(activate(z, act));
+}
+
 }  // namespace mll
 
 using namespace mll;
@@ -425,13 +438,13 @@ const char* mll_last_error() { return g_error.c_str(); }
 int mll_version() { return 1; }
 
 int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float* out,
-                  int n_tokens, int width, int vocab, hipStream_t stream) {
+                  int n_tokens, int width, int vocab, float scale, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && width > 0 && vocab > 0, "embedding: sizes must be positive");
     if (n_tokens == 0) return 0;
     if (table_dtype == kF32) {
-        embedding_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids, out, width, vocab);
+        embedding_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids, out, width, vocab, scale);
     } else if (table_dtype == kBF16) {
-        embedding_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids, out, width, vocab);
+        embedding_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids, out, width, vocab, scale);
     } else {
         return fail("embedding: unknown table dtype");
     }
@@ -483,6 +496,25 @@ int mll_add_bias(float* values, const float* bias, int64_t n_rows, int width, hi
     MLL_REQUIRE(blocks < (1ll << 31), "add_bias: too many values for one launch");
     add_bias_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(values, bias, count, width);
     return check_launch("add_bias");
+}
+
+int mll_activation(const void* in, int in_dtype, int n_parts, int64_t part_stride, void* out, int dtype, int64_t count, int act,
+                   hipStream_t stream) {
+    MLL_REQUIRE(act >= 0 && act <= 2, "activation: 0 SiLU, 1 gelu (erf), 2 gelu (tanh)");
+    MLL_REQUIRE(n_parts >= 1, "activation: at least one part");
+    if (count <= 0) return 0;
+    const int64_t blocks = (count + 255) / 256;
+    MLL_REQUIRE(blocks < (1ll << 31), "activation: too many values for one launch");
+    const unsigned grid = static_cast<unsigned>(blocks);
+    if (in_dtype == kF32 && dtype == kF32)
+        activation_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<const float*>(in), n_parts, part_stride, static_cast<float*>(out), count, act);
+    else if (in_dtype == kF32 && dtype == kBF16)
+        activation_kernel<bf16, float><<<grid, 256, 0, stream>>>(static_cast<const float*>(in), n_parts, part_stride, static_cast<bf16*>(out), count, act);
+    else if (in_dtype == kBF16 && dtype == kBF16)
+        activation_kernel<bf16, bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(in), n_parts, part_stride, static_cast<bf16*>(out), count, act);
+    else
+        return fail("activation: the input is float32 or has the output's type");
+    return check_launch("activation");
 }
 
 int mll_softcap(float* values, int64_t count, float cap, hipStream_t stream) {

@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(kWave)
 gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
                 const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
                 const int32_t* __restrict__ slots, float* __restrict__ out, int heads, int key_dim, int value_dim,
-                int lanes_a_column, float q_scale) {
+                int lanes_a_column, float q_scale, int64_t decay_stride) {
     __shared__ float lane_sums[kWave];
     const int seq = blockIdx.x;
     const int head = blockIdx.y;
@@ -69,7 +69,7 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
     float a_next[ROWS], k_next[ROWS], q_next[ROWS], v_next;
     auto fetch = [&](int token) {
         const float* row = proj + static_cast<int64_t>(token) * proj_stride;
-        const float* decays = decay + static_cast<int64_t>(token) * channels + head * key_dim;
+        const float* decays = decay + static_cast<int64_t>(token) * decay_stride + head * key_dim;
 #pragma unroll
         for (int m = 0; m < ROWS; ++m) {
             const int i = ROWS * r + m;
@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(kWave)
 gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
                       const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
                       const int32_t* __restrict__ slots, float* __restrict__ out, int heads, int key_dim, int value_dim,
-                      int lanes_a_column, int tile_tokens, float q_scale) {
+                      int lanes_a_column, int tile_tokens, float q_scale, int64_t decay_stride) {
     __shared__ __align__(16) float buffer_even[kScanBufferFloats];
     __shared__ __align__(16) float buffer_odd[kScanBufferFloats];
     __shared__ __align__(16) float lane_sums[64 * kWave];    // of a tile's tokens (at most 64), added up after its walk
@@ -175,7 +175,7 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
             const int64_t token = min(tile_first + token_of[j], last - 1);
             constexpr int kPiece = WIDE ? 4 : 1;
             const float* row = proj + token * proj_stride + head * key_dim + channel_of[j];
-            const float* decays = decay + token * channels + head * key_dim + channel_of[j];
+            const float* decays = decay + token * decay_stride + head * key_dim + channel_of[j];
             float* place = buffer + j * kWave * kPiece;
             if constexpr (WIDE) {
                 __builtin_amdgcn_global_load_lds(decays, place, 16, 0, 0);
@@ -261,7 +261,7 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     }
 }
 
-// out[t, head, :] = rms_norm(o[t, head, :]) * weight * silu(gate[t, head, :]) * out_scale; one wave a (token, head).
+// out[t, head, :] = rms_norm(o[t, head, :]) * weight * silu(gate[t, head, :]) * out_scale (weight null: none); one wave a (token, head).
 template <typename T>
 __global__ void __launch_bounds__(kWave)
 gla_gate_kernel(const float* __restrict__ o, const float* __restrict__ proj, int64_t proj_stride, int gate_offset,
@@ -279,7 +279,7 @@ gla_gate_kernel(const float* __restrict__ o, const float* __restrict__ proj, int
     for (int c = lane; c < value_dim; c += kWave) {
         const float g = gate[c];
         const float silu = g / (1.0f + expf(-g));
-        to[c] = from_float<T>(row[c] * factor * weight[c] * silu * out_scale);
+        to[c] = from_float<T>((weight ? row[c] * factor * weight[c] : row[c] * factor) * silu * out_scale);
     }
 }
 
@@ -310,12 +310,14 @@ int mll_gla_decay(const float* proj, int64_t proj_stride, int low_offset, int ra
 
 int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset, const float* decay,
                  float* state, const int32_t* cu_tokens, const int32_t* slots, float* out, int n_seqs, int heads, int key_dim,
-                 int value_dim, float q_scale, int long_portions, hipStream_t stream) {
+                 int value_dim, float q_scale, int long_portions, int64_t decay_stride, hipStream_t stream) {
     MLL_REQUIRE(n_seqs >= 0 && heads > 0 && key_dim > 0 && value_dim > 0, "gla_scan: sizes must be positive");
     MLL_REQUIRE(key_dim <= kWideHeadRows * kWave, "gla_scan: key heads wider than 512 are not supported");
     MLL_REQUIRE(q_offset >= 0 && k_offset >= 0 && v_offset >= 0 && q_offset + heads * key_dim <= proj_stride &&
                     k_offset + heads * key_dim <= proj_stride && v_offset + heads * value_dim <= proj_stride,
                 "gla_scan: a projection lies outside its row");
+    MLL_REQUIRE(decay_stride == 0 || decay_stride >= static_cast<int64_t>(heads) * key_dim,
+                "gla_scan: the decays of a token are heads * key_dim numbers; a stride of 0 gives every token the same");
     if (n_seqs == 0) return 0;
     const int rows = key_dim <= kUsualRows * kWave ? kUsualRows : kWideHeadRows;
     int lanes_a_column = 1;
@@ -329,11 +331,12 @@ int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_off
         if (tile_tokens * columns_a_wave > kScanTileFloats) tile_tokens = kScanTileFloats / columns_a_wave;
         if (tile_tokens > 64) tile_tokens = 64;
         const bool wide = key_dim % 8 == 0 && proj_stride % 4 == 0 && q_offset % 4 == 0 && k_offset % 4 == 0 &&
-                          reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(decay) % 16 == 0;
+                          reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(decay) % 16 == 0 &&
+                          decay_stride % 4 == 0;
 #define MLL_SCAN_TILED(WIDE, ROWS)                                                                                         \
     gla_scan_tiled_kernel<WIDE, ROWS><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, \
                                                                  cu_tokens, slots, out, heads, key_dim, value_dim,              \
-                                                                 lanes_a_column, tile_tokens, q_scale)
+                                                                 lanes_a_column, tile_tokens, q_scale, decay_stride)
         if (wide && rows == kUsualRows) MLL_SCAN_TILED(true, kUsualRows);
         else if (wide) MLL_SCAN_TILED(true, kWideHeadRows);
         else if (rows == kUsualRows) MLL_SCAN_TILED(false, kUsualRows);
@@ -343,10 +346,10 @@ int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_off
     }
     if (rows == kUsualRows) {
         gla_scan_kernel<kUsualRows><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
-                                                               slots, out, heads, key_dim, value_dim, lanes_a_column, q_scale);
+                                                               slots, out, heads, key_dim, value_dim, lanes_a_column, q_scale, decay_stride);
     } else {
         gla_scan_kernel<kWideHeadRows><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
-                                                                  slots, out, heads, key_dim, value_dim, lanes_a_column, q_scale);
+                                                                  slots, out, heads, key_dim, value_dim, lanes_a_column, q_scale, decay_stride);
     }
     return check_launch("gla_scan");
 }

@@ -13,9 +13,14 @@ extern "C" {
 const char* mll_last_error();
 int mll_version();
 
-// out[t, :] = table[ids[t], :] widened to float32. An id outside [0, vocab) gives a row of NaN.
+// out[t, :] = table[ids[t], :] widened to float32, times scale. An id outside [0, vocab) gives a row of NaN.
 int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float* out,
-                  int n_tokens, int width, int vocab, hipStream_t stream);
+                  int n_tokens, int width, int vocab, float scale, hipStream_t stream);
+
+// out[i] = act(in[i]) for count values; in is float32 (n_parts partial sums part_stride elements apart, added in
+// order first) or of the output's type. act: 0 SiLU, 1 the exact gelu 0.5 z (1 + erf(z / sqrt 2)), 2 the tanh form.
+int mll_activation(const void* in, int in_dtype, int n_parts, int64_t part_stride, void* out, int dtype, int64_t count, int act,
+                   hipStream_t stream);
 
 // For i < n_rows, r = rows ? rows[i] : i:  v = h[r] + (delta ? delta[r] : 0);
 // if write_h, h[r] = v;  out[i] = v * rsqrt(mean(v^2) + eps) * weight.
@@ -28,10 +33,11 @@ int mll_rms_norm(float* h, const void* delta, int delta_dtype, int n_partials, i
 
 // d = the delta's parts added in order; v = h[r] + mult * d * rsqrt(mean(d^2) + after_eps) * after_weight; if write_h,
 // h[r] = v; out[i] = v * rsqrt(mean(v^2) + eps) * weight (weight null: no output). A sublayer's result that is normed
-// itself before it joins the stream, fused with the norm that follows (csrc/norm_after.hip).
+// itself before it joins the stream, fused with the norm that follows (csrc/norm_after.hip). extra (null: none): float32
+// rows like h's, added to v after the delta (what a model adds to its stream between two layers).
 int mll_rms_norm_after(float* h, const void* delta, int delta_dtype, int n_partials, int64_t partial_stride,
-                       const int32_t* rows, const float* after_weight, float after_eps, float mult, const float* weight,
-                       float eps, void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream);
+                       const int32_t* rows, const float* after_weight, float after_eps, float mult, const float* extra,
+                       const float* weight, float eps, void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream);
 
 // values[r][c] += bias[c] for n_rows rows of `width` float32 values, in place.
 int mll_add_bias(float* values, const float* bias, int64_t n_rows, int width, hipStream_t stream);
@@ -289,21 +295,27 @@ int mll_clamped_glu(const float* gate_up, void* out, int dtype, int n_tokens, in
 // (temp_coef 0: not). Queries go to q_out [t][heads][key_dim]; keys and values into the pages
 // [slot][kv_head][dim] at slot_mapping[t] (negative: not stored), or, with tiled_page_size > 0 (the positions of a
 // page; key_dim == value_dim), into pages in the MFMA kernels' order (cache_layout.h).
+// Rows of qkv lie row_stride floats apart (they may hold further columns after the values). With cos_sin (float32
+// [n_tokens][rot_dims / 2][cos, sin]) queries and keys are turned after their norm: channel i < rot_dims / 2 of a head
+// with channel i + rot_dims / 2, (u, v) -> (u cos - v sin, v cos + u sin); the other channels pass.
 int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const float* q_weight, const float* k_weight,
                       float eps, const int32_t* positions, const int32_t* slot_mapping, float temp_coef, int temp_every,
                       void* q_out, void* k_pages, void* v_pages, int dtype, int n_tokens, int heads, int kv_heads, int key_dim,
-                      int value_dim, int tiled_page_size, const float* bias, int normed, int queries_only, hipStream_t stream);
+                      int value_dim, int tiled_page_size, const float* bias, int normed, int queries_only, int64_t row_stride,
+                      const float* cos_sin, int rot_dims, hipStream_t stream);
 
 // Causal attention of every token over its request's pages: score_j = (q . k_j) * scale + bias[min(p - j, longest)][head]
 // (bias null: none; float32 [longest + 1][heads]) - slopes[head] * (p - j) (slopes null: none); softmax over j <= p
 // (with window > 0: p - window < j <= p) with exp(sink[head]) added to the denominator
 // (sink null: not); out[t][head] = out_scale * sum_j weight_j v_j, rows out_stride elements apart.
 // A token whose seq_of_token is negative is skipped. The order of every sum depends on p alone.
+// With chunk > 0 (and no window) a query at p sees the keys from floor(p / chunk) * chunk on. With gate (float32, rows
+// gate_stride apart, one number a head) the head's result is multiplied by sigmoid(gate[t][head]).
 int mll_bias_attention(const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_width,
                        const int32_t* seq_of_token, const int32_t* positions, const float* bias, int longest,
                        const float* sink, void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int kv_heads,
                        int key_dim, int value_dim, int page_size, float scale, float out_scale, const float* slopes, int window,
-                       hipStream_t stream);
+                       int chunk, const float* gate, int64_t gate_stride, hipStream_t stream);
 
 // ---- gated linear attention --------------------------------------------------------------------------------
 
@@ -317,12 +329,13 @@ int mll_gla_decay(const float* proj, int64_t proj_stride, int low_offset, int ra
 // q, k, v are float32 columns of proj's rows at the given offsets. A request without tokens is passed over.
 // long_portions: the kernel that brings tiles of tokens through LDS (for steps with portions of many tokens); the
 // same operations per token in the same order either way, so the same bits.
+// decay: float32, token t's heads * key_dim numbers at decay + t * decay_stride (0: one row for every token).
 int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset, const float* decay,
                  float* state, const int32_t* cu_tokens, const int32_t* slots, float* out, int n_seqs, int heads, int key_dim,
-                 int value_dim, float q_scale, int long_portions, hipStream_t stream);
+                 int value_dim, float q_scale, int long_portions, int64_t decay_stride, hipStream_t stream);
 
 // out[t][head] = o[t][head] / rms(o[t][head]) * weight * silu(gate[t][head]) * out_scale, gate at gate_offset of
-// proj's rows; out in `dtype`, rows out_stride elements apart.
+// proj's rows (weight null: none); out in `dtype`, rows out_stride elements apart.
 int mll_gla_gate(const float* o, const float* proj, int64_t proj_stride, int gate_offset, const float* weight, float eps,
                  void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int value_dim, float out_scale,
                  hipStream_t stream);
@@ -414,13 +427,17 @@ int mll_rglru_scan(const float* proj, int64_t proj_stride, int x_at, const float
 // ids[t][n], weights[t][n] for n < top: the experts with the largest scores (sigmoid, or softmax over the experts)
 // of z[t][0 .. experts), ties to the lower index; weights are the scores, divided by their sum with renormalize.
 // shared_at >= 0: shared_gate[t] = sigmoid(z[t][shared_at]).
+// groups > 0: the experts form that many equal groups of neighbours; a group's score is its largest, and only experts of
+// the `keep` best groups (ties: the lower) are chosen.
 int mll_moe_route(const float* z, int64_t z_stride, int n_tokens, int experts, int top, int softmax_scores, int renormalize,
-                  int shared_at, int32_t* ids, float* weights, float* shared_gate, hipStream_t stream);
+                  int shared_at, int32_t* ids, float* weights, float* shared_gate, int groups, int keep, hipStream_t stream);
 
 // act[t * top + n] = silu(Wg_e xs) * (Wu_e xs), e = ids[t][n], xs = x[t] * weights[t][n] rounded to `dtype`
 // (weight_on_input) or x[t]; gate_up [experts][2 * ff][width] with the gate rows first.
+// gated 0: gate_up is [experts][ff][width] and act = activation(Wu_e xs). activation: 0 SiLU, 1 gelu (erf), 2 gelu (tanh).
 int mll_moe_gate_up(const void* x, const int32_t* ids, const float* weights, int top, const void* gate_up, void* act,
-                    int dtype, int n_tokens, int width, int ff, int weight_on_input, hipStream_t stream);
+                    int dtype, int n_tokens, int width, int ff, int weight_on_input, int gated, int activation,
+                    hipStream_t stream);
 
 // out[n][t] = Wd_e act[t * top + n] (* weights[t][n] unless weight_on_input): float32 [top][n_tokens][width].
 int mll_moe_down(const void* act, const int32_t* ids, const float* weights, int top, const void* down, float* out, int dtype,
@@ -440,7 +457,7 @@ int mll_scale_rows(const float* in, int n_parts, int64_t part_stride, const floa
 // width and ff are multiples of 8.
 int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int top, const void* gate_up, const void* down,
                     int32_t* counts, int32_t* offsets, int32_t* order, void* sorted, void* act, float* out, int n_tokens,
-                    int experts, int width, int ff, int weight_on_input, hipStream_t stream);
+                    int experts, int width, int ff, int weight_on_input, int gated, int activation, hipStream_t stream);
 
 // mll_rglru_scan for steps with long portions: the recurrence in chunks of 64 tokens (every chunk walked from zero,
 // the state carried from chunk to chunk, every chunk walked again from its start), the same result but for the

@@ -1,5 +1,6 @@
 // A mixture of experts: the choice of every token's experts from router logits, and the experts' gated
-// feed-forwards for (token, choice) pairs whose expert is only known on the device.
+// feed-forwards for (token, choice) pairs whose expert is only known on the device. An expert is gated,
+// Wd (act(Wg x) * (Wu x)), or has one inner weight, Wd act(Wu x); act is chosen by number (common.h).
 //
 // Choice: scores are sigmoid(z) or softmax(z) over the experts, the `top` largest are taken (ties: the lower
 // index), their weights are the scores, optionally divided by their sum. Everything float32.
@@ -20,7 +21,7 @@ constexpr int kMaxTop = 16;
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const float* __restrict__ z, int64_t z_stride, int n_tokens, int experts, int top, int softmax_scores,
                  int renormalize, int shared_at, int32_t* __restrict__ ids, float* __restrict__ weights,
-                 float* __restrict__ shared_gate) {
+                 float* __restrict__ shared_gate, int groups, int keep) {
     const int token = blockIdx.x * blockDim.x + threadIdx.x;
     if (token >= n_tokens) return;
     const float* row = z + static_cast<int64_t>(token) * z_stride;
@@ -29,6 +30,27 @@ moe_route_kernel(const float* __restrict__ z, int64_t z_stride, int n_tokens, in
         for (int e = 0; e < experts; ++e) peak = fmaxf(peak, row[e]);
         total = 0.0f;
         for (int e = 0; e < experts; ++e) total += expf(row[e] - peak);
+    }
+    // Groups of neighbouring experts: a group counts as much as its best expert, and only the experts of the `keep`
+    // best groups (ties: the lower group) can be chosen. A bit a group (at most 64).
+    unsigned long long open_groups = ~0ull;
+    const int group_size = groups > 0 ? experts / groups : experts;
+    if (groups > 0 && keep < groups) {
+        open_groups = 0ull;
+        for (int n = 0; n < keep; ++n) {
+            int best_group = -1;
+            float best_logit = 0.0f;
+            for (int g = 0; g < groups; ++g) {
+                if ((open_groups >> g) & 1ull) continue;
+                float top_logit = row[g * group_size];
+                for (int e = 1; e < group_size; ++e) top_logit = fmaxf(top_logit, row[g * group_size + e]);
+                if (best_group < 0 || top_logit > best_logit) {
+                    best_group = g;
+                    best_logit = top_logit;
+                }
+            }
+            open_groups |= 1ull << best_group;
+        }
     }
     int chosen[kMaxTop];
     float taken[kMaxTop];
@@ -39,7 +61,7 @@ moe_route_kernel(const float* __restrict__ z, int64_t z_stride, int n_tokens, in
         for (int e = 0; e < experts; ++e) {
             bool used = false;
             for (int m = 0; m < n; ++m) used = used || chosen[m] == e;
-            if (used) continue;
+            if (used || (groups > 0 && !((open_groups >> (e / group_size)) & 1ull))) continue;
             // the scores rise with the logits, so the largest logit is the largest score; a logit that is no number is never larger
             if (best < 0 || row[e] > best_logit) {
                 best = e;
@@ -156,7 +178,8 @@ constexpr int kExpertRowsABlock = kExpertWaves * kExpertRowsAWave;
 template <typename T>
 __global__ void __launch_bounds__(kExpertWaves * kWave)
 moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids, const float* __restrict__ weights, int top,
-                   const T* __restrict__ gate_up, T* __restrict__ act, int width, int ff, int weight_on_input) {
+                   const T* __restrict__ gate_up, T* __restrict__ act, int width, int ff, int weight_on_input, int gated,
+                   int activation) {
     extern __shared__ float xs[];
     const int pair = blockIdx.y;
     const int token = pair / top;
@@ -166,6 +189,23 @@ moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids, con
         xs[c] = to_float(from_float<T>(to_float(x[static_cast<int64_t>(token) * width + c]) * factor));
     __syncthreads();
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    if (!gated) {       // act[pair][f] = activation(Wu_e[f] . xs); gate_up is [experts][ff][width]
+        const T* up = gate_up + static_cast<int64_t>(expert) * ff * width;
+        for (int n = 0; n < kExpertRowsAWave; n += 4) {
+            const int f = blockIdx.x * kExpertRowsABlock + wave * kExpertRowsAWave + n;
+            if (f >= ff) break;
+            const T* const rows[4] = {up + static_cast<int64_t>(f) * width, up + static_cast<int64_t>(min(f + 1, ff - 1)) * width,
+                                      up + static_cast<int64_t>(min(f + 2, ff - 1)) * width, up + static_cast<int64_t>(min(f + 3, ff - 1)) * width};
+            float sums[4];
+            rows_dot4<T>(rows, xs, width, lane, sums);
+            if (lane == 0) {
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    if (f + m < ff) act[static_cast<int64_t>(pair) * ff + f + m] = from_float<T>(activate(sums[m], activation));
+            }
+        }
+        return;
+    }
     const T* base = gate_up + static_cast<int64_t>(expert) * 2 * ff * width;
     for (int n = 0; n < kExpertRowsAWave; n += 2) {      // two outputs at a time: their gate and up rows are four rows
         const int f = blockIdx.x * kExpertRowsABlock + wave * kExpertRowsAWave + n;
@@ -176,8 +216,8 @@ moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids, con
         float sums[4];
         rows_dot4<T>(rows, xs, width, lane, sums);
         if (lane == 0) {
-            act[static_cast<int64_t>(pair) * ff + f] = from_float<T>(sums[0] / (1.0f + expf(-sums[0])) * sums[1]);
-            if (f + 1 < ff) act[static_cast<int64_t>(pair) * ff + f + 1] = from_float<T>(sums[2] / (1.0f + expf(-sums[2])) * sums[3]);
+            act[static_cast<int64_t>(pair) * ff + f] = from_float<T>(activate(sums[0], activation) * sums[1]);
+            if (f + 1 < ff) act[static_cast<int64_t>(pair) * ff + f + 1] = from_float<T>(activate(sums[2], activation) * sums[3]);
         }
     }
 }
@@ -283,15 +323,17 @@ moe_gather_kernel(const bf16* __restrict__ x, const int32_t* __restrict__ order,
 
 constexpr int kGroupRows = 128, kGroupCols = 128, kGroupStep = 64, kGroupPad = 72;     // rows of a tile lie 144 bytes apart in LDS: 16-byte reads of 16 rows meet no bank twice
 
-// GATED: w is [experts][2 * n_half][k] (gate rows, then up rows); a tile holds 64 gate rows and the 64 up rows that
+// FORM 2: w is [experts][n_out][k] and out (bfloat16 [pairs][n_out], sorted order) gets activation(product).
+// FORM 1 (GATED): w is [experts][2 * n_half][k] (gate rows, then up rows); a tile holds 64 gate rows and the 64 up rows that
 // belong to them, and out (bfloat16 [pairs][n_half], sorted order) gets silu(gate) * up. Otherwise w is
 // [experts][n_out][k] and out (float32 [top][n_tokens][n_out]) gets the product at the pair's token and choice,
 // times the pair's weight unless that multiplied the input.
-template <bool GATED>
+template <int FORM>
 __global__ void __launch_bounds__(256)
 moe_grouped_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w, const int32_t* __restrict__ offsets,
                    const int32_t* __restrict__ order, const float* __restrict__ weights, int experts, int n_out, int k,
-                   void* __restrict__ out, int top, int n_tokens, int weight_on_input) {
+                   void* __restrict__ out, int top, int n_tokens, int weight_on_input, int activation) {
+    constexpr bool GATED = FORM == 1;
     __shared__ __attribute__((aligned(16))) bf16 a_tile[kGroupRows * kGroupPad];
     __shared__ __attribute__((aligned(16))) bf16 w_tile[kGroupCols * kGroupPad];
     int expert = 0, first_row = 0, rows = 0, before = 0;
@@ -392,7 +434,16 @@ moe_grouped_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w, const
                 for (int i = 0; i < 4; ++i) {
                     const int column = col0 + wn * 32 + nt * 16 + quad * 4 + i;
                     const float g = acc[mt][nt][i], u = acc[mt][nt + 2][i];
-                    if (column < n_out) to[column] = from_float<bf16>(g / (1.0f + expf(-g)) * u);
+                    if (column < n_out) to[column] = from_float<bf16>(activate(g, activation) * u);
+                }
+        } else if (FORM == 2) {
+            bf16* to = static_cast<bf16*>(out) + static_cast<int64_t>(first_row + row) * n_out;
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int column = col0 + w_base[nt] + quad * 4 + i;
+                    if (column < n_out) to[column] = from_float<bf16>(activate(acc[mt][nt][i], activation));
                 }
         } else {
             const int pair = order[first_row + row];
@@ -416,19 +467,24 @@ using namespace mll;
 extern "C" {
 
 int mll_moe_route(const float* z, int64_t z_stride, int n_tokens, int experts, int top, int softmax_scores, int renormalize,
-                  int shared_at, int32_t* ids, float* weights, float* shared_gate, hipStream_t stream) {
+                  int shared_at, int32_t* ids, float* weights, float* shared_gate, int groups, int keep, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && experts > 0 && top > 0 && top <= experts, "moe_route: 1 <= top <= experts");
     MLL_REQUIRE(top <= kMaxTop, "moe_route: more than 16 experts a token are not supported");
     MLL_REQUIRE(shared_at < 0 || shared_gate != nullptr, "moe_route: the shared expert's gate needs a place");
+    MLL_REQUIRE(groups == 0 || (groups > 0 && groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups &&
+                                keep * (experts / groups) >= top),
+                "moe_route: at most 64 equal groups, of which the kept ones hold at least `top` experts");
     if (n_tokens == 0) return 0;
     moe_route_kernel<<<(n_tokens + 63) / 64, 64, 0, stream>>>(z, z_stride, n_tokens, experts, top, softmax_scores, renormalize,
-                                                            shared_at, ids, weights, shared_gate);
+                                                            shared_at, ids, weights, shared_gate, groups, keep);
     return check_launch("moe_route");
 }
 
 int mll_moe_gate_up(const void* x, const int32_t* ids, const float* weights, int top, const void* gate_up, void* act,
-                    int dtype, int n_tokens, int width, int ff, int weight_on_input, hipStream_t stream) {
+                    int dtype, int n_tokens, int width, int ff, int weight_on_input, int gated, int activation,
+                    hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && top > 0 && width > 0 && ff > 0, "moe_gate_up: sizes must be positive");
+    MLL_REQUIRE(activation >= 0 && activation <= 2, "moe_gate_up: 0 SiLU, 1 gelu (erf), 2 gelu (tanh)");
     MLL_REQUIRE(static_cast<int64_t>(n_tokens) * top < 65536, "moe_gate_up: too many (token, expert) pairs for one launch");
     MLL_REQUIRE(static_cast<size_t>(width) * sizeof(float) <= 64 * 1024, "moe_gate_up: rows wider than 16384 are not supported");
     if (n_tokens == 0) return 0;
@@ -436,10 +492,10 @@ int mll_moe_gate_up(const void* x, const int32_t* ids, const float* weights, int
     const size_t lds = static_cast<size_t>(width) * sizeof(float);
     if (dtype == kF32) {
         moe_gate_up_kernel<float><<<grid, kExpertWaves * kWave, lds, stream>>>(
-            static_cast<const float*>(x), ids, weights, top, static_cast<const float*>(gate_up), static_cast<float*>(act), width, ff, weight_on_input);
+            static_cast<const float*>(x), ids, weights, top, static_cast<const float*>(gate_up), static_cast<float*>(act), width, ff, weight_on_input, gated, activation);
     } else if (dtype == kBF16) {
         moe_gate_up_kernel<bf16><<<grid, kExpertWaves * kWave, lds, stream>>>(
-            static_cast<const bf16*>(x), ids, weights, top, static_cast<const bf16*>(gate_up), static_cast<bf16*>(act), width, ff, weight_on_input);
+            static_cast<const bf16*>(x), ids, weights, top, static_cast<const bf16*>(gate_up), static_cast<bf16*>(act), width, ff, weight_on_input, gated, activation);
     } else {
         return fail("moe_gate_up: unknown dtype");
     }
@@ -482,8 +538,9 @@ int mll_scale_rows(const float* in, int n_parts, int64_t part_stride, const floa
 
 int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int top, const void* gate_up, const void* down,
                     int32_t* counts, int32_t* offsets, int32_t* order, void* sorted, void* act, float* out, int n_tokens,
-                    int experts, int width, int ff, int weight_on_input, hipStream_t stream) {
+                    int experts, int width, int ff, int weight_on_input, int gated, int activation, hipStream_t stream) {
     MLL_REQUIRE(n_tokens > 0 && top > 0 && experts > 0 && width > 0 && ff > 0, "moe_grouped: sizes must be positive");
+    MLL_REQUIRE(activation >= 0 && activation <= 2, "moe_grouped: 0 SiLU, 1 gelu (erf), 2 gelu (tanh)");
     MLL_REQUIRE(width % 8 == 0 && ff % 8 == 0, "moe_grouped: widths must be multiples of 8");
     const int64_t pairs = static_cast<int64_t>(n_tokens) * top;
     MLL_REQUIRE(pairs < (1 << 30), "moe_grouped: too many (token, expert) pairs");
@@ -494,12 +551,18 @@ int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int
                                                   weight_on_input);
     const int tiles = (n_pairs + kGroupRows - 1) / kGroupRows + experts;
     MLL_REQUIRE(tiles < 65536, "moe_grouped: too many tiles of rows for one launch");
-    moe_grouped_kernel<true><<<dim3((ff + 63) / 64, tiles), 256, 0, stream>>>(
-        static_cast<const bf16*>(sorted), static_cast<const bf16*>(gate_up), offsets, order, weights, experts, ff, width, act, top,
-        n_tokens, weight_on_input);
-    moe_grouped_kernel<false><<<dim3((width + kGroupCols - 1) / kGroupCols, tiles), 256, 0, stream>>>(
+    if (gated) {
+        moe_grouped_kernel<1><<<dim3((ff + 63) / 64, tiles), 256, 0, stream>>>(
+            static_cast<const bf16*>(sorted), static_cast<const bf16*>(gate_up), offsets, order, weights, experts, ff, width, act, top,
+            n_tokens, weight_on_input, activation);
+    } else {
+        moe_grouped_kernel<2><<<dim3((ff + kGroupCols - 1) / kGroupCols, tiles), 256, 0, stream>>>(
+            static_cast<const bf16*>(sorted), static_cast<const bf16*>(gate_up), offsets, order, weights, experts, ff, width, act, top,
+            n_tokens, weight_on_input, activation);
+    }
+    moe_grouped_kernel<0><<<dim3((width + kGroupCols - 1) / kGroupCols, tiles), 256, 0, stream>>>(
         static_cast<const bf16*>(act), static_cast<const bf16*>(down), offsets, order, weights, experts, width, ff, out, top, n_tokens,
-        weight_on_input);
+        weight_on_input, activation);
     return check_launch("moe_grouped");
 }
 

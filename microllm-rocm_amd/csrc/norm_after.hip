@@ -1,7 +1,7 @@
 // A sublayer's result that is RMS-normed itself before it joins the residual stream, and the norm that follows:
 //
 //   d = sum of the delta's parts, in order          (the partial sums of a product cut along its reduction)
-//   v = h + mult * d * rsqrt(mean(d^2) + after_eps) * after_weight
+//   v = h + mult * d * rsqrt(mean(d^2) + after_eps) * after_weight (+ extra, a further float32 row for every row of h)
 //   out = v * rsqrt(mean(v^2) + eps) * weight       (weight null: no output, the sum alone)
 //
 // One workgroup a row; the row stays in registers between the two sums of squares. Both sums are float32 and
@@ -17,7 +17,7 @@ template <typename T, typename D, int CHUNKS>
 __global__ void __launch_bounds__(kAfterThreads)
 rms_norm_after_kernel(float* __restrict__ h, const D* __restrict__ delta, int n_partials, int64_t partial_stride,
                       const int32_t* __restrict__ rows, const float* __restrict__ after_weight, float after_eps, float mult,
-                      const float* __restrict__ weight, float eps, T* __restrict__ out, int width, int write_h) {
+                      const float* __restrict__ extra, const float* __restrict__ weight, float eps, T* __restrict__ out, int width, int write_h) {
     __shared__ float scratch[16];
     const int index = blockIdx.x;
     const int64_t source = rows ? rows[index] : index;
@@ -42,7 +42,8 @@ rms_norm_after_kernel(float* __restrict__ h, const D* __restrict__ delta, int n_
     for (int c = 0; c < CHUNKS; ++c) {
         const int column = threadIdx.x + c * kAfterThreads;
         if (column < width) {
-            const float value = h_row[column] + d[c] * after * after_weight[column];
+            float value = h_row[column] + d[c] * after * after_weight[column];
+            if (extra) value += extra[source * width + column];
             d[c] = value;
             if (write_h) h_row[column] = value;
             squares = fmaf(value, value, squares);
@@ -69,7 +70,7 @@ __device__ inline float4 after_load_four(const bf16* source) {
 template <typename T, typename D, int CHUNKS>
 __global__ void rms_norm_after_vec4_kernel(float* __restrict__ h, const D* __restrict__ delta, int n_partials, int64_t partial_stride,
                                            const int32_t* __restrict__ rows, const float* __restrict__ after_weight, float after_eps,
-                                           float mult, const float* __restrict__ weight, float eps, T* __restrict__ out, int width,
+                                           float mult, const float* __restrict__ extra, const float* __restrict__ weight, float eps, T* __restrict__ out, int width,
                                            int write_h) {
     __shared__ float scratch[16];
     const int index = blockIdx.x;
@@ -120,6 +121,13 @@ __global__ void rms_norm_after_vec4_kernel(float* __restrict__ h, const D* __res
             value.y = stream[c].y + d[c].y * after * w.y;
             value.z = stream[c].z + d[c].z * after * w.z;
             value.w = stream[c].w + d[c].w * after * w.w;
+            if (extra) {
+                const float4 more = reinterpret_cast<const float4*>(extra + source * width)[q];
+                value.x += more.x;
+                value.y += more.y;
+                value.z += more.z;
+                value.w += more.w;
+            }
             d[c] = value;
             if (write_h) reinterpret_cast<float4*>(h_row)[q] = value;
             squares = fmaf(value.x, value.x, squares);
@@ -146,26 +154,27 @@ __global__ void rms_norm_after_vec4_kernel(float* __restrict__ h, const D* __res
 
 template <typename T, typename D>
 static int launch_after(float* h, const D* delta, int n_partials, int64_t partial_stride, const int32_t* rows,
-                        const float* after_weight, float after_eps, float mult, const float* weight, float eps, T* out,
+                        const float* after_weight, float after_eps, float mult, const float* extra, const float* weight, float eps, T* out,
                         int n_rows, int width, int write_h, hipStream_t stream) {
 #define MLL_AFTER(CHUNKS)                                                                                                \
     rms_norm_after_kernel<T, D, CHUNKS><<<n_rows, kAfterThreads, 0, stream>>>(h, delta, n_partials, partial_stride, rows, \
-                                                                              after_weight, after_eps, mult, weight, eps, \
+                                                                              after_weight, after_eps, mult, extra, weight, eps, \
                                                                               out, width, write_h)
     const bool delta_aligned = sizeof(D) != sizeof(float) ||
                                (reinterpret_cast<uintptr_t>(delta) % 16 == 0 && (n_partials == 1 || partial_stride % 4 == 0));
     const bool aligned = width % 4 == 0 && delta_aligned && reinterpret_cast<uintptr_t>(h) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(after_weight) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0;
+                         reinterpret_cast<uintptr_t>(after_weight) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(extra) % 16 == 0;
     const int quads = width / 4;
     if (aligned && quads <= 1024) {
         const int threads = quads <= 64 ? 64 : (quads + 63) / 64 * 64;
         rms_norm_after_vec4_kernel<T, D, 1><<<n_rows, threads, 0, stream>>>(h, delta, n_partials, partial_stride, rows, after_weight,
-                                                                           after_eps, mult, weight, eps, out, width, write_h);
+                                                                           after_eps, mult, extra, weight, eps, out, width, write_h);
         return check_launch("rms_norm_after");
     }
     if (aligned && quads <= 4096) {
         rms_norm_after_vec4_kernel<T, D, 4><<<n_rows, 1024, 0, stream>>>(h, delta, n_partials, partial_stride, rows, after_weight,
-                                                                        after_eps, mult, weight, eps, out, width, write_h);
+                                                                        after_eps, mult, extra, weight, eps, out, width, write_h);
         return check_launch("rms_norm_after");
     }
     const int chunks = (width + kAfterThreads - 1) / kAfterThreads;
@@ -186,7 +195,7 @@ using namespace mll;
 
 extern "C" int mll_rms_norm_after(float* h, const void* delta, int delta_dtype, int n_partials, int64_t partial_stride,
                                   const int32_t* rows, const float* after_weight, float after_eps, float mult,
-                                  const float* weight, float eps, void* out, int dtype, int n_rows, int width, int write_h,
+                                  const float* extra, const float* weight, float eps, void* out, int dtype, int n_rows, int width, int write_h,
                                   hipStream_t stream) {
     MLL_REQUIRE(h != nullptr && delta != nullptr && after_weight != nullptr, "rms_norm_after: a stream, a delta and its norm's weight");
     MLL_REQUIRE(n_partials >= 1, "rms_norm_after: the delta needs at least one part");
@@ -197,12 +206,12 @@ extern "C" int mll_rms_norm_after(float* h, const void* delta, int delta_dtype, 
     if (n_rows == 0) return 0;
     if (dtype == kF32 && delta_dtype == kF32)
         return launch_after<float, float>(h, static_cast<const float*>(delta), n_partials, partial_stride, rows, after_weight,
-                                          after_eps, mult, weight, eps, static_cast<float*>(out), n_rows, width, write_h, stream);
+                                          after_eps, mult, extra, weight, eps, static_cast<float*>(out), n_rows, width, write_h, stream);
     if (dtype == kBF16 && delta_dtype == kF32)
         return launch_after<bf16, float>(h, static_cast<const float*>(delta), n_partials, partial_stride, rows, after_weight,
-                                         after_eps, mult, weight, eps, static_cast<bf16*>(out), n_rows, width, write_h, stream);
+                                         after_eps, mult, extra, weight, eps, static_cast<bf16*>(out), n_rows, width, write_h, stream);
     if (dtype == kBF16 && delta_dtype == kBF16)
         return launch_after<bf16, bf16>(h, static_cast<const bf16*>(delta), n_partials, partial_stride, rows, after_weight,
-                                        after_eps, mult, weight, eps, static_cast<bf16*>(out), n_rows, width, write_h, stream);
+                                        after_eps, mult, extra, weight, eps, static_cast<bf16*>(out), n_rows, width, write_h, stream);
     return fail("rms_norm_after: the delta is float32 or has the output's type");
 }

@@ -59,7 +59,8 @@ def _device_tensor(tensor: torch.Tensor, name: str, dtype: Optional[torch.dtype]
     _need(tensor.dtype == dtype, f"{name} must be {dtype}, got {tensor.dtype}")
 
 
-def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """``table[ids] * scale`` as float32 rows."""
     lib = library.load()
     _device_tensor(table, "embedding table")
     _device_tensor(ids, "token ids", torch.int32)
@@ -70,7 +71,7 @@ def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor
     _device_tensor(out, "embedding output", torch.float32)
     _need(tuple(out.shape) == (ids.shape[0], width), "embedding output has the wrong shape")
     _check(lib.mll_embedding(_ptr(table), _code(table.dtype), _ptr(ids), _ptr(out),
-                             ids.shape[0], width, vocab, _stream()), lib)
+                             ids.shape[0], width, vocab, ctypes.c_float(scale), _stream()), lib)
     return out
 
 
@@ -112,10 +113,10 @@ def rms_norm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch
 
 def rms_norm_after(h: torch.Tensor, delta: torch.Tensor, after_weight: torch.Tensor, after_eps: float, mult: float,
                    weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
-                   write_h: bool = False) -> Optional[torch.Tensor]:
+                   write_h: bool = False, extra: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """``v = h[rows] + mult * rms_norm(delta[rows]) * after_weight`` (``delta`` may be float32 partial sums ``[parts,
-    tokens, width]``, added in order first); with ``write_h`` the sum replaces ``h``; returns ``rms_norm(v) * weight``,
-    or None without ``weight``."""
+    tokens, width]``, added in order first), plus ``extra[rows]`` (float32 rows like ``h``'s) if given; with ``write_h`` the
+    sum replaces ``h``; returns ``rms_norm(v) * weight``, or None without ``weight``."""
     lib = library.load()
     _device_tensor(h, "residual stream", torch.float32)
     _device_tensor(after_weight, "norm weight of the delta", torch.float32)
@@ -135,13 +136,16 @@ def rms_norm_after(h: torch.Tensor, delta: torch.Tensor, after_weight: torch.Ten
         n_rows = rows.shape[0]
     else:
         n_rows = h.shape[0]
+    if extra is not None:
+        _device_tensor(extra, "further rows for the stream", torch.float32)
+        _need(tuple(extra.shape) == tuple(h.shape), "the further rows must have the residual stream's shape")
     out = None
     if weight is not None:
         _device_tensor(weight, "norm weight", torch.float32)
         _need(tuple(weight.shape) == (width,), "the norm weight must match the stream's width")
         out = torch.empty((n_rows, width), dtype=out_dtype, device=h.device)
     _check(lib.mll_rms_norm_after(_ptr(h), _ptr(delta), _code(delta.dtype), n_partials, ctypes.c_int64(h.numel()), _ptr(rows),
-                                  _ptr(after_weight), ctypes.c_float(after_eps), ctypes.c_float(mult), _ptr(weight),
+                                  _ptr(after_weight), ctypes.c_float(after_eps), ctypes.c_float(mult), _ptr(extra), _ptr(weight),
                                   ctypes.c_float(eps), _ptr(out), _code(out_dtype), n_rows, width, int(write_h), _stream()), lib)
     return out
 
@@ -163,6 +167,27 @@ def softcap(values: torch.Tensor, cap: float) -> torch.Tensor:
     _device_tensor(values, "values", torch.float32)
     _check(lib.mll_softcap(_ptr(values), ctypes.c_int64(values.numel()), ctypes.c_float(cap), _stream()), lib)
     return values
+
+
+ACTIVATIONS = {"silu": 0, "gelu_erf": 1, "gelu_tanh": 2}
+
+
+def activation(values: torch.Tensor, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
+    """``act(values)`` element by element in ``out_dtype``; ``values`` is float32 (then it may be partial sums ``[parts,
+    rows, width]``, added in order first) or has ``out_dtype``. ``kind``: ``silu``, ``gelu_erf`` (the exact gelu) or
+    ``gelu_tanh``."""
+    lib = library.load()
+    _device_tensor(values, "values")
+    _need(kind in ACTIVATIONS, f"unknown activation {kind!r}")
+    _need(values.dtype in (torch.float32, out_dtype), "the values are float32 or have the output's dtype")
+    n_parts, part_stride = 1, 0
+    if values.dim() == 3:
+        _need(values.dtype == torch.float32, "partial sums are float32")
+        n_parts, part_stride = values.shape[0], values.shape[1] * values.shape[2]
+    out = torch.empty(tuple(values.shape[-2:]) if values.dim() == 3 else tuple(values.shape), dtype=out_dtype, device=values.device)
+    _check(lib.mll_activation(_ptr(values), _code(values.dtype), n_parts, ctypes.c_int64(part_stride), _ptr(out), _code(out_dtype),
+                              ctypes.c_int64(out.numel()), ACTIVATIONS[kind], _stream()), lib)
+    return out
 
 
 def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
@@ -1095,7 +1120,7 @@ def embedding_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.
     _need(tuple(rates.shape) == ((width + 1) // 2,), "one rate per pair of columns")
     out = torch.empty((ids.shape[0], width), dtype=torch.float32, device=table.device)
     _check(lib.mll_embedding_sinusoid(_ptr(table), _code(table.dtype), _ptr(ids), _ptr(positions), _ptr(rates), _ptr(out),
-                                      ids.shape[0], width, vocab, _stream()), lib)
+                                      ids.shape[0], width, vocab, ctypes.c_float(scale), _stream()), lib)
     return out
 
 
@@ -1191,18 +1216,28 @@ def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight:
                   positions: torch.Tensor, slot_mapping: torch.Tensor, temp_coef: float, temp_every: int,
                   k_pages: torch.Tensor, v_pages: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int,
                   out_dtype: torch.dtype, tiled_page_size: int = 0, bias: Optional[torch.Tensor] = None,
-                  normed: Optional[bool] = None, queries_only: bool = False) -> torch.Tensor:
+                  normed: Optional[bool] = None, queries_only: bool = False, cos_sin: Optional[torch.Tensor] = None,
+                  further_columns: int = 0) -> torch.Tensor:
     """Norm of queries and keys over their head, the queries' factor by position, keys and values into their pages
     (``[page, position, kv_head, dim]``, or with ``tiled_page_size`` the pages of ``cache.layout`` with that many
     positions each); returns the queries ``[tokens, heads * key_dim]``. ``bias`` (one number a column of a row) is
     added first. ``normed`` (by default: where weights are given) divides queries and keys by their root mean square
     also without weights. With ``queries_only`` the rows hold queries alone and nothing is stored (a layer that
-    reads another's keys and values)."""
+    reads another's keys and values). With ``cos_sin`` (``rope_table``'s ``[tokens, n, 2]``) queries and keys are turned
+    after their norm in their first ``2 n`` channels, channel ``i`` with ``i + n``. The rows may hold
+    ``further_columns`` after the values (what another kernel reads from the same product)."""
     lib = library.load()
     n_parts, part_stride = _parts_of(qkv, "q/k/v")
     n_tokens = qkv.shape[-2]
     row_width = heads * key_dim if queries_only else (heads + kv_heads) * key_dim + kv_heads * value_dim
-    _need(qkv.shape[-1] == row_width, "q/k/v rows have the wrong width")
+    _need(qkv.shape[-1] == row_width + further_columns, "q/k/v rows have the wrong width")
+    row_stride = ctypes.c_int64(qkv.shape[-1])
+    rot_dims = 0
+    if cos_sin is not None:
+        _device_tensor(cos_sin, "cos and sin of the positions", torch.float32)
+        _need(cos_sin.dim() == 3 and cos_sin.shape[0] >= n_tokens and cos_sin.shape[2] == 2 and 2 * cos_sin.shape[1] <= key_dim,
+              "cos and sin are [tokens, pairs, 2] with at most key_dim / 2 pairs")
+        rot_dims = 2 * cos_sin.shape[1]
     _device_tensor(positions, "positions", torch.int32)
     _need(positions.shape[0] >= n_tokens, "a position for every token")
     if normed is None:
@@ -1217,7 +1252,8 @@ def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight:
         _check(lib.mll_qk_norm_store(_ptr(qkv), n_parts, ctypes.c_int64(part_stride), _ptr(q_weight), _ptr(q_weight),
                                      ctypes.c_float(eps), _ptr(positions), None, ctypes.c_float(temp_coef),
                                      int(temp_every), _ptr(q_out), None, None, _code(out_dtype), n_tokens,
-                                     heads, kv_heads, key_dim, value_dim, 0, _ptr(bias), int(normed), 1, _stream()), lib)
+                                     heads, kv_heads, key_dim, value_dim, 0, _ptr(bias), int(normed), 1, row_stride, _ptr(cos_sin),
+                                     rot_dims, _stream()), lib)
         return q_out
     _device_tensor(slot_mapping, "slot mapping", torch.int32)
     _need(slot_mapping.shape[0] >= n_tokens, "a slot for every token")
@@ -1238,7 +1274,7 @@ def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight:
                                  ctypes.c_float(eps), _ptr(positions), _ptr(slot_mapping), ctypes.c_float(temp_coef),
                                  int(temp_every), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _code(out_dtype), n_tokens,
                                  heads, kv_heads, key_dim, value_dim, int(tiled_page_size), _ptr(bias), int(normed), 0,
-                                 _stream()), lib)
+                                 row_stride, _ptr(cos_sin), rot_dims, _stream()), lib)
     return q_out
 
 
@@ -1246,10 +1282,12 @@ def bias_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
                    seq_of_token: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor],
                    sink: Optional[torch.Tensor], scale: float, out_scale: float, heads: int, kv_heads: int, key_dim: int,
                    value_dim: int, out: Optional[torch.Tensor] = None, slopes: Optional[torch.Tensor] = None,
-                   window: int = 0) -> torch.Tensor:
+                   window: int = 0, chunk: int = 0, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention with ``bias[min(distance, last row), head]`` added to the scaled scores, ``slopes[head] *
     distance`` taken off them, and ``exp(sink[head])`` in the softmax's denominator; with ``window`` a query sees
-    itself and the ``window - 1`` keys before it; ``out`` may be columns of a wider buffer (its row stride is taken)."""
+    itself and the ``window - 1`` keys before it; with ``chunk`` the keys from ``floor(p / chunk) * chunk`` on; with ``gate``
+    (float32 ``[tokens, heads]``, columns of a wider buffer allowed) a head's result is multiplied by ``sigmoid(gate)``;
+    ``out`` may be columns of a wider buffer (its row stride is taken)."""
     lib = library.load()
     _device_tensor(q, "queries")
     n_tokens = q.shape[0]
@@ -1276,7 +1314,12 @@ def bias_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
     if slopes is not None:
         _device_tensor(slopes, "slopes", torch.float32)
         _need(tuple(slopes.shape) == (heads,), "one slope a head")
-    _need(window >= 0, "a window is positive, or 0 for none")
+    _need(window >= 0 and chunk >= 0 and not (window and chunk), "a window or chunks of positions (0 for none), not both")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and tuple(gate.shape) == (n_tokens, heads)
+              and gate.stride(1) == 1, "the gate is float32 [tokens, heads] with unit column stride")
+        gate_stride = max(gate.stride(0), heads)
     if out is None:
         out = torch.empty((n_tokens, heads * value_dim), dtype=q.dtype, device=q.device)
     _need(out.is_cuda and out.dtype == q.dtype and out.dim() == 2 and tuple(out.shape) == (n_tokens, heads * value_dim)
@@ -1285,7 +1328,8 @@ def bias_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor
                                   _ptr(seq_of_token), _ptr(positions), _ptr(bias), longest, _ptr(sink),
                                   ctypes.c_void_p(out.data_ptr()), ctypes.c_int64(out.stride(0) if n_tokens > 1 else max(out.stride(0), heads * value_dim)),
                                   _code(q.dtype), n_tokens, heads, kv_heads, key_dim, value_dim, page_size,
-                                  ctypes.c_float(scale), ctypes.c_float(out_scale), _ptr(slopes), int(window), _stream()), lib)
+                                  ctypes.c_float(scale), ctypes.c_float(out_scale), _ptr(slopes), int(window), int(chunk),
+                                  ctypes.c_void_p(gate.data_ptr()) if gate is not None else None, ctypes.c_int64(gate_stride), _stream()), lib)
     return out
 
 
@@ -1323,25 +1367,28 @@ def gla_scan(proj: torch.Tensor, q_offset: int, k_offset: int, v_offset: int, de
     _device_tensor(cu_tokens, "token offsets", torch.int32)
     _device_tensor(slots, "state slots", torch.int32)
     n_tokens = proj.shape[0]
-    _need(proj.dim() == 2 and tuple(decay.shape) == (n_tokens, heads * key_dim), "decays are [tokens, heads * key_dim]")
+    _need(proj.dim() == 2 and tuple(decay.shape) in ((n_tokens, heads * key_dim), (heads * key_dim,)),
+          "decays are [tokens, heads * key_dim], or [heads * key_dim] for every token alike")
+    decay_stride = heads * key_dim if decay.dim() == 2 else 0
     _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, key_dim, value_dim), "state is [slots, heads, key_dim, value_dim]")
     _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
     out = torch.empty((n_tokens, heads * value_dim), dtype=torch.float32, device=proj.device)
     _check(lib.mll_gla_scan(_ptr(proj), ctypes.c_int64(proj.shape[1]), q_offset, k_offset, v_offset, _ptr(decay), _ptr(state),
                             _ptr(cu_tokens), _ptr(slots), _ptr(out), n_seqs, heads, key_dim, value_dim,
-                            ctypes.c_float(q_scale), int(long_portions), _stream()), lib)
+                            ctypes.c_float(q_scale), int(long_portions), ctypes.c_int64(decay_stride), _stream()), lib)
     return out
 
 
-def gla_gate(o: torch.Tensor, proj: torch.Tensor, gate_offset: int, weight: torch.Tensor, eps: float, heads: int,
+def gla_gate(o: torch.Tensor, proj: torch.Tensor, gate_offset: int, weight: Optional[torch.Tensor], eps: float, heads: int,
              value_dim: int, out_scale: float, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Per head: ``o / rms(o) * weight * silu(gate) * out_scale``; ``out`` may be columns of a wider buffer."""
+    """Per head: ``o / rms(o) * weight * silu(gate) * out_scale`` (``weight`` None: none); ``out`` may be columns of a wider buffer."""
     lib = library.load()
     _device_tensor(o, "recurrence output", torch.float32)
     _device_tensor(proj, "projections", torch.float32)
-    _device_tensor(weight, "norm weight", torch.float32)
+    if weight is not None:
+        _device_tensor(weight, "norm weight", torch.float32)
     n_tokens = o.shape[0]
-    _need(tuple(o.shape) == (n_tokens, heads * value_dim) and proj.shape[0] == n_tokens and tuple(weight.shape) == (value_dim,),
+    _need(tuple(o.shape) == (n_tokens, heads * value_dim) and proj.shape[0] == n_tokens and (weight is None or tuple(weight.shape) == (value_dim,)),
           "gla_gate takes [tokens, heads * value_dim], the projections of the same tokens and a weight [value_dim]")
     if out is None:
         out = torch.empty((n_tokens, heads * value_dim), dtype=out_dtype, device=o.device)
@@ -1650,9 +1697,11 @@ def router_logits(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
 
 
 def moe_route(z: torch.Tensor, experts: int, top: int, softmax_scores: bool = False, renormalize: bool = False,
-              shared_at: int = -1):
+              shared_at: int = -1, groups: int = 0, keep: int = 0):
     """The ``top`` experts of every token from router logits ``z`` float32 ``[tokens, columns]`` (experts first):
-    ``(ids int32 [tokens, top], weights float32 [tokens, top], sigmoid(z[:, shared_at]) or None)``."""
+    ``(ids int32 [tokens, top], weights float32 [tokens, top], sigmoid(z[:, shared_at]) or None)``. With ``groups``
+    the experts form that many equal groups of neighbours, a group counts as its best expert, and only experts of the
+    ``keep`` best groups are chosen."""
     lib = library.load()
     _device_tensor(z, "router logits", torch.float32)
     _need(z.dim() == 2 and z.shape[1] >= experts and shared_at < z.shape[1], "router logits are [tokens, experts (+ gate)]")
@@ -1661,7 +1710,7 @@ def moe_route(z: torch.Tensor, experts: int, top: int, softmax_scores: bool = Fa
     weights = torch.empty((n_tokens, top), dtype=torch.float32, device=z.device)
     shared = torch.empty((n_tokens,), dtype=torch.float32, device=z.device) if shared_at >= 0 else None
     _check(lib.mll_moe_route(_ptr(z), ctypes.c_int64(z.shape[1]), n_tokens, experts, top, int(softmax_scores), int(renormalize),
-                             int(shared_at), _ptr(ids), _ptr(weights), _ptr(shared), _stream()), lib)
+                             int(shared_at), _ptr(ids), _ptr(weights), _ptr(shared), int(groups), int(keep), _stream()), lib)
     return ids, weights, shared
 
 
@@ -1672,12 +1721,14 @@ MOE_GROUPED_PAIRS = 64      # from this many (token, choice) pairs on, bfloat16 
 
 
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
-                weight_on_input: bool, out: Optional[torch.Tensor] = None, grouped: Optional[bool] = None) -> torch.Tensor:
+                weight_on_input: bool, out: Optional[torch.Tensor] = None, grouped: Optional[bool] = None, gated: bool = True,
+                activation: str = "silu") -> torch.Tensor:
     """Every (token, choice) pair through its expert's gated feed-forward: ``gate_up`` ``[experts, 2 * ff, width]``
     (gate rows first), ``down`` ``[experts, width, ff]``. Returns float32 ``[top, tokens, width]``, a part per choice,
     for the reader to add in order (``out``: at least that many leading parts of a larger buffer). ``grouped``: the
     pairs sorted by expert and multiplied in tiles on the matrix units (bfloat16, widths in steps of 8) instead of
-    one reading of the expert's weights a pair; by default by the number of pairs."""
+    one reading of the expert's weights a pair; by default by the number of pairs. With ``gated`` false an expert is
+    ``down act(up x)`` and ``gate_up`` holds ``[experts, ff, width]``; ``activation`` is one of ``ACTIVATIONS``."""
     lib = library.load()
     _device_tensor(x, "expert input")
     _device_tensor(gate_up, "experts' gate and up weights", x.dtype)
@@ -1686,8 +1737,10 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_
     _device_tensor(weights, "expert weights", torch.float32)
     n_tokens, width = x.shape
     top = ids.shape[1]
-    experts, double, _ = gate_up.shape
-    ff = double // 2
+    experts, inner_rows, _ = gate_up.shape
+    ff = inner_rows // 2 if gated else inner_rows
+    _need(activation in ACTIVATIONS, f"unknown activation {activation!r}")
+    act_code = ACTIVATIONS[activation]
     _need(gate_up.shape[2] == width and tuple(down.shape) == (experts, width, ff) and tuple(ids.shape) == (n_tokens, top)
           and tuple(weights.shape) == (n_tokens, top), "the experts' weights, ids and weights do not fit the input")
     if out is None:
@@ -1704,7 +1757,7 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_
         in_order = torch.empty((n_tokens * top, width), dtype=x.dtype, device=x.device)
         _check(lib.mll_moe_grouped(_ptr(x), _ptr(ids), _ptr(weights), top, _ptr(gate_up), _ptr(down), ctypes.c_void_p(counts.data_ptr()),
                                    ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()), _ptr(in_order), _ptr(act),
-                                   _ptr(out), n_tokens, experts, width, ff, int(weight_on_input), _stream()), lib)
+                                   _ptr(out), n_tokens, experts, width, ff, int(weight_on_input), int(gated), act_code, _stream()), lib)
         return out
     step = max(1, MOE_PAIRS_A_LAUNCH // top)       # tokens a launch: its grid has a row of workgroups a pair
     element = x.element_size()
@@ -1713,7 +1766,7 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_
         here = dict(x=ctypes.c_void_p(x.data_ptr() + first * width * element), ids=ctypes.c_void_p(ids.data_ptr() + first * top * 4),
                     weights=ctypes.c_void_p(weights.data_ptr() + first * top * 4), act=ctypes.c_void_p(act.data_ptr() + first * top * ff * element))
         _check(lib.mll_moe_gate_up(here["x"], here["ids"], here["weights"], top, _ptr(gate_up), here["act"], _code(x.dtype), count, width, ff,
-                                   int(weight_on_input), _stream()), lib)
+                                   int(weight_on_input), int(gated), act_code, _stream()), lib)
         # the output keeps its rows n_tokens apart in every part: the launch writes its tokens' rows of each
         _check(lib.mll_moe_down_rows(here["act"], here["ids"], here["weights"], top, _ptr(down), ctypes.c_void_p(out.data_ptr() + first * width * 4),
                                      _code(x.dtype), count, n_tokens, width, ff, int(weight_on_input), _stream()), lib)

@@ -92,9 +92,24 @@ class LatentAttention(Mixer):
             decls[self.name("g")] = TensorDecl((self.gate_width, self.hidden), MATRIX)
         return decls
 
+    def _turned_rows_reordered(self, weight: torch.Tensor, vectors: int, first: int, stride: int) -> torch.Tensor:
+        """``weight``'s rows that make the turned parts (``vectors`` runs of ``rot_dim`` rows, the first at ``first``,
+        ``stride`` apart) brought into the order the position encoding turns them in."""
+        order = self.position.split_half_order().to(weight.device)
+        rows = torch.arange(weight.shape[0], device=weight.device)
+        for vector in range(vectors):
+            at = first + vector * stride
+            rows[at:at + self.rot_dim] = at + order
+        return weight[rows].contiguous()
+
     def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
         roles = ["dq" if self.q_rank else "q"] + (["dkv"] if self.owns_kv else []) + (["g"] if self.output_gate else [])
         weights = [tensors[self.name(role)] for role in roles]
+        reorder = hasattr(self.position, "split_half_order")     # queries' and keys' turned channels, both alike
+        if reorder and not self.q_rank:
+            weights[0] = self._turned_rows_reordered(weights[0], self.heads, self.dim, self.dim + self.rot_dim)
+        if reorder and self.owns_kv:
+            weights[1] = self._turned_rows_reordered(weights[1], 1, self.kv_rank, 0)
         if len({w.dtype for w in weights}) != 1:
             raise TypeError("the projections of one layer must share a dtype to be stacked")
         keep = self.runtime.keep_plain_weights
@@ -102,7 +117,10 @@ class LatentAttention(Mixer):
         del weights
         self.o_weight = Weight(tensors[self.name("o")], keep_plain=keep)
         if self.q_rank:
-            self.uq_weight = Weight(tensors[self.name("uq")], keep_plain=keep)
+            uq = tensors[self.name("uq")]
+            if reorder:
+                uq = self._turned_rows_reordered(uq, self.heads, self.dim, self.dim + self.rot_dim)
+            self.uq_weight = Weight(uq, keep_plain=keep)
             self.q_norm = tensors[self.name("dq_norm")]
         if self.owns_kv:
             self.kv_norm = tensors[self.name("dkv_norm")]

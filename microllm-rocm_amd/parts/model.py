@@ -14,14 +14,16 @@ import torch
 from ..ops import kernels
 from .base import CacheNeed, MATRIX, Part, Runtime, TensorDecl
 from .block import Block, build_block
-from .linear import Weight, linear
+from .linear import UnscaledRows, Weight, linear
+from .norm import NormedDelta
 from .registry import build_part, register_part
 from .spec import ModelSpec, PartSpec
 
 
 class TokenEmbedding(Part):
-    """``h0[t] = E[id_t]`` widened to float32 (src/model/model.cpp:1111). An embedding part is handed the whole
-    step, so that one which also needs positions or requests (learned positions, token types) finds them."""
+    """``h0[t] = E[id_t]`` widened to float32 (src/model/model.cpp:1111), times ``scale`` if the spec gives one. An
+    embedding part is handed the whole step, so that one which also needs positions or requests (learned positions,
+    token types) finds them."""
     category = "embedding"
     graph_safe = True
 
@@ -29,6 +31,7 @@ class TokenEmbedding(Part):
         super().__init__(spec, runtime)
         self.vocab = int(spec.params["vocab_size"])
         self.width = int(spec.params["hidden_size"])
+        self.scale = float(spec.params.get("scale", 1.0))
         self.table: Optional[torch.Tensor] = None
 
     def tensors(self):
@@ -38,7 +41,7 @@ class TokenEmbedding(Part):
         self.table = tensors[self.name("weight")]
 
     def forward(self, ctx) -> torch.Tensor:
-        return kernels.embedding(self.table, ctx.tokens)
+        return kernels.embedding(self.table, ctx.tokens, scale=self.scale)
 
     def bytes_read(self, rows: int, context: int) -> int:
         return rows * self.width * self.table.element_size()     # a row per token, not the table
@@ -170,6 +173,20 @@ class Model:
         return needs
 
     # ---- forward -------------------------------------------------------------------------
+    @staticmethod
+    def _add_to_stream(h: torch.Tensor, pending, rows: torch.Tensor):
+        """``h + pending + rows`` before the next entry: a delta that is still to be normed takes the rows along, so
+        that the norm which reads the stream next adds both in its one kernel; anything else is added here."""
+        if isinstance(pending, NormedDelta):
+            return pending.with_extra(rows)
+        if h.dim() != 2 or isinstance(pending, UnscaledRows):
+            raise TypeError("rows join a single residual stream that no product has already summed and normed")
+        if pending is not None:
+            pending = pending.to(torch.float32)
+            kernels.residual_add(h, pending.sum(0) if pending.dim() == 3 else pending)
+        kernels.residual_add(h, rows)
+        return None
+
     def forward(self, ctx, caches, want_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
         """Run the step's tokens through every entry; logits ``[wanted, vocab]`` in float32.
 
@@ -181,8 +198,12 @@ class Model:
             h = kernels.stream_copies(h, self.spec.streams)
         pending = None
         order = self.spec.order
+        # the embedding's output once more, for the entries before which it joins the stream again (h is written over)
+        again = self.embedding.forward(ctx) if any(entry.adds_embedding for entry in order) else None
         for index, entry in enumerate(order):
             next_block = self.blocks[order[index + 1].layer] if index + 1 < len(order) else None
+            if entry.adds_embedding:
+                pending = self._add_to_stream(h, pending, again)
             pending = self.blocks[entry.layer].forward(h, pending, ctx, caches[index], next_block)
             if self.observer is not None:
                 self.observer(index, h, pending)

@@ -20,19 +20,27 @@ class NormedDelta:
     """A sublayer's result that is still to be RMS-normed with a weight of its own and multiplied by ``mult`` before
     it joins the residual stream: ``h += mult * values / sqrt(mean(values^2) + eps) * weight``. The norm that reads the
     stream next does both in one kernel. ``values`` is ``[tokens, hidden]`` or float32 partial sums ``[parts, tokens,
-    hidden]``, which are added in order first."""
+    hidden]``, which are added in order first. ``extra``: float32 rows ``[tokens, hidden]`` that join the stream after
+    it, unnormed (``with_extra``)."""
 
-    def __init__(self, values: torch.Tensor, weight: torch.Tensor, eps: float, mult: float):
+    def __init__(self, values: torch.Tensor, weight: torch.Tensor, eps: float, mult: float, extra: Optional[torch.Tensor] = None):
         self.values = values
         self.weight = weight
         self.eps = float(eps)
         self.mult = float(mult)
+        self.extra = extra
+
+    def with_extra(self, rows: torch.Tensor) -> "NormedDelta":
+        if self.extra is not None:
+            raise ValueError("this delta already takes further rows along")
+        return NormedDelta(self.values, self.weight, self.eps, self.mult, rows)
 
     def resolved(self) -> torch.Tensor:
         """What joins the stream, as a float32 tensor ``[tokens, hidden]`` (for observers; a step never needs it)."""
         shape = self.values.shape[-2:]
         joined = torch.zeros(shape, dtype=torch.float32, device=self.values.device)
-        kernels.rms_norm_after(joined, self.values, self.weight, self.eps, self.mult, None, 1.0, self.values.dtype, write_h=True)
+        kernels.rms_norm_after(joined, self.values, self.weight, self.eps, self.mult, None, 1.0, self.values.dtype, write_h=True,
+                               extra=self.extra)
         return joined
 
 
@@ -61,7 +69,7 @@ class RMSNorm(Norm):
     def forward(self, h, delta=None, write_h=True, rows=None):
         if isinstance(delta, NormedDelta):
             return kernels.rms_norm_after(h, delta.values, delta.weight, delta.eps, delta.mult, self.weight, self.eps,
-                                          self.runtime.dtype, rows=rows, write_h=write_h and rows is None)
+                                          self.runtime.dtype, rows=rows, write_h=write_h and rows is None, extra=delta.extra)
         return kernels.rms_norm(h, self.weight, self.eps, self.runtime.dtype, delta=delta, rows=rows,
                                 write_h=write_h and delta is not None and rows is None)
 

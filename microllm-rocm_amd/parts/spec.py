@@ -45,9 +45,13 @@ class RunEntry:
     ``layer`` indexes ``ModelSpec.layers`` and may appear in several entries
     (shared weights; each entry has a cache of its own). ``reads_cache_of`` names
     an earlier entry whose cache this entry's mixer reads instead of owning one.
+    With ``adds_embedding`` the embedding's output joins the residual stream once
+    more right before this entry (a model that runs a range of layers several
+    times and feeds its input in again at every pass).
     """
     layer: int
     reads_cache_of: Optional[int] = None
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)
