@@ -117,6 +117,27 @@ def zabozen_config(size: dict):
     return ZabozenConfig(vocab=DESIGN_VOCAB, width=width, norm_eps=1e-6, residual_mult=0.5, layers=tuple(layers), logit_softcap=30.0)
 
 
+def kalevik_config(size: dict):
+    """A Kalevik configuration of the given layer sizes: layers in turn a latent attention (heads of 96 unrotated and 64
+    rotated query/key dims and 128 value dims, cached rows of 192 + 64 elements) with a dense feed-forward, and a parallel
+    mixer (a softmax attention of the model's heads and key/value heads inside chunks of 8192 positions, which a
+    prompt of 2048 tokens and a context of 4096 lie within, so that it reads every key as Qwen2's does, half of every
+    head turned; beside it a retention of half as many heads with keys of half the head size, as Siditar's linear
+    attention) with 16 experts of a quarter of the feed-forward width, four a token out of the best two of four groups,
+    and a shared expert of half of it. Every layer runs once: a looped range is the same layers again."""
+    from microllm_rocm_amd.config.kalevik import (ChunkAttentionConfig, DenseMlpConfig, KalevikConfig, KalevikLayerConfig,
+                                                  LatentAttentionConfig, MoeMlpConfig, ParallelConfig, RetentionConfig)
+    width, heads, kv_heads, dim, ff = size["width"], size["heads"], size["kv_heads"], size["head_dim"], size["ff"]
+    latent = LatentAttentionConfig(heads=heads, dim=96, rot_dim=64, vdim=dim, kv_rank=192, scale=160 ** -0.5, rot_base=1e6, rot_dims=64)
+    left = ChunkAttentionConfig(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, chunk=8192, rot_base=1e6,
+                                rot_dims=dim // 2, rot_factor=4.0)
+    right = RetentionConfig(heads=heads // 2, dim=dim // 2, vdim=dim, decay=tuple(1.0 - 2.0 ** (-5 - head % 6) for head in range(heads // 2)))
+    moe = MoeMlpConfig(experts=16, top=4, expert_ff=ff // 4, groups=4, keep_groups=2, shared_ff=ff // 2)
+    layers = [KalevikLayerConfig("latent_attention", latent, DenseMlpConfig(ff)) if index % 2 == 0 else
+              KalevikLayerConfig("parallel", ParallelConfig(left, right, 0.6, 0.9), moe) for index in range(size["layers"])]
+    return KalevikConfig(vocab=DESIGN_VOCAB, width=width, norm_eps=1e-6, layers=tuple(layers), embedding_scale=3.0)
+
+
 def design_configs(size: dict, design: str = "siditar"):
     """The design's configuration at the given layer sizes and the Qwen2 configuration of equal width, heads, head size,
     feed-forward width, depth and vocabulary."""
@@ -129,6 +150,9 @@ def design_configs(size: dict, design: str = "siditar"):
         return {"gupitar": gupitar_config(size), "qwen2": qwen2}
     if design == "zabozen":     # beside the design whose layers are most like its own, and beside Qwen2
         return {"zabozen": zabozen_config(size), "gupitar": gupitar_config(size), "qwen2": qwen2}
+    if design == "kalevik":     # beside the designs whose layers are most like its own (latents and experts; a parallel mixer)
+        return {"kalevik": kalevik_config(size), "gupitar": gupitar_config(size), "siditar": design_configs(size, "siditar")["siditar"],
+                "qwen2": qwen2}
     from microllm_rocm_amd.config.siditar import (BiasAttentionConfig, DenseMlpConfig, LinearAttentionConfig,
                                                   ParallelMixerConfig, SiditarConfig, SiditarLayerConfig)
     left = BiasAttentionConfig(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["head_dim"], vdim=size["head_dim"],
@@ -208,11 +232,11 @@ def main() -> int:
     parser.add_argument("--no-extras", action="store_true",
                         help="leave out what the default run adds to its line after the main figures: decoding on the 32-bit path "
                              "at batch 8 and the continuous-batching workload at Qwen2-0.5B sizes")
-    parser.add_argument("--design", default=None, choices=["siditar", "gupitar", "zabozen"],
+    parser.add_argument("--design", default=None, choices=["siditar", "gupitar", "zabozen", "kalevik"],
                         help="instead of the default workload: prefill and decode throughput of this design beside Qwen2 at equal "
                              "layer sizes (--design-sizes), random weights; --batch, --context, --prefill-tokens, --steps apply")
     parser.add_argument("--design-sizes", default="1k,2k,4k", help="of " + ", ".join(sorted(DESIGN_SIZES)))
-    parser.add_argument("--design-only", default=None, choices=["siditar", "gupitar", "zabozen", "qwen2"], help="one of the designs alone (profiles)")
+    parser.add_argument("--design-only", default=None, choices=["siditar", "gupitar", "zabozen", "kalevik", "qwen2"], help="one of the designs alone (profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")

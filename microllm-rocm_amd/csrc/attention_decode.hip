@@ -40,9 +40,16 @@ union Frag8 {
     uint4 raw;
 };
 
+// The factor of a head's gate on its result: sigmoid(gate[token][head]), or 1 without a gate.
+__device__ inline float head_gate(const MllAttentionExtras& extras, int token, int head) {
+    if (extras.gate == nullptr) return 1.0f;
+    return 1.0f / (1.0f + __expf(-extras.gate[static_cast<int64_t>(token) * extras.gate_stride + head]));
+}
+
 // EXTRA: the scores also get extras.bias[min(position - key, longest)][head], the softmax's denominator also holds
 // exp(extras.sink[head]) (counted once, where the waves' or the splits' results meet), the result is multiplied by
-// extras.out_scale and its rows lie extras.out_stride elements apart. Without EXTRA the kernel is what it was.
+// extras.out_scale and by the head's gate and its rows lie extras.out_stride elements apart; with extras.chunk the keys
+// seen begin at the query's chunk of positions. Without EXTRA the kernel is what it was.
 template <int HD_TILES, bool STREAM, bool EXTRA>
 __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
@@ -78,7 +85,8 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
 
     const int seq = seq_of_token[token];
     const int position = positions[token];
-    const int low = window > 0 ? max(0, position - window + 1) : 0;
+    // the oldest key seen: the first of the query's chunk of positions, or what the window reaches back to
+    const int low = (EXTRA && extras.chunk > 0) ? position / extras.chunk * extras.chunk : (window > 0 ? max(0, position - window + 1) : 0);
     const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;
 
     const int first_pair = low / 32, last_pair = position / 32;
@@ -297,7 +305,7 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
         const int64_t row = static_cast<int64_t>(token) * heads + head0 + h;
         const int64_t part_row = static_cast<int64_t>(blockIdx.x) * heads + head0 + h;   // partial results are kept densely
         if (n_splits == 1) {
-            if (EXTRA) out[static_cast<int64_t>(token) * extras.out_stride + (head0 + h) * HD + dim] = from_float<bf16>(total / sum * extras.out_scale);
+            if (EXTRA) out[static_cast<int64_t>(token) * extras.out_stride + (head0 + h) * HD + dim] = from_float<bf16>(total / sum * extras.out_scale * head_gate(extras, token, head0 + h));
             else out[row * HD + dim] = from_float<bf16>(total / sum);
         } else {
             part_o[(part_row * n_splits + split) * HD + dim] = total;
@@ -351,7 +359,7 @@ __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, co
             }
         }
         if (with_sink) weight_sum += __expf(sink - top);
-        if (EXTRA) out[static_cast<int64_t>(token) * extras.out_stride + (blockIdx.x % heads) * head_dim + dim] = from_float<bf16>(total / weight_sum * extras.out_scale);
+        if (EXTRA) out[static_cast<int64_t>(token) * extras.out_stride + (blockIdx.x % heads) * head_dim + dim] = from_float<bf16>(total / weight_sum * extras.out_scale * head_gate(extras, token, blockIdx.x % heads));
         else out[row * head_dim + dim] = from_float<bf16>(total / weight_sum);
     }
 }

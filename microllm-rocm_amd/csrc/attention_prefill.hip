@@ -115,13 +115,18 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
 
     // Either tile's tokens and the keys any of them can see (tokens of a portion have consecutive positions);
     // an empty tile sees nothing: no key lies in its range.
+    // the oldest key a token at `position` sees: the first of its chunk of positions, or what the window reaches back to
+    auto low_of = [&](int position) {
+        if (EXTRA && extras.chunk > 0) return position / extras.chunk * extras.chunk;
+        return window > 0 ? max(0, position - window + 1) : 0;
+    };
     int range_low[2], range_last[2], tile_positions[2];
 #pragma unroll
     for (int side = 0; side < 2; ++side) {
         const int count = entry[2 + 2 * side];
         tile_positions[side] = count > 0 ? positions[entry[1 + 2 * side]] : 0;
         range_last[side] = count > 0 ? tile_positions[side] + count - 1 : -1;
-        range_low[side] = count > 0 ? (window > 0 ? max(0, tile_positions[side] - window + 1) : 0) : (1 << 30);
+        range_low[side] = count > 0 ? low_of(tile_positions[side]) : (1 << 30);
     }
     const int group_low = min(range_low[0], range_low[1]);
     const int group_last = max(range_last[0], range_last[1]);
@@ -151,11 +156,11 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     const int block_valid = min(32, max(0, count - block_first));
     const int block_position = tile_position + block_first;
     const int block_last = block_position + block_valid - 1;
-    const int block_low = window > 0 ? max(0, block_position - window + 1) : 0;        // the lowest key its first token sees
-    const int block_last_low = window > 0 ? max(0, block_last - window + 1) : 0;       // and its last token
+    const int block_low = low_of(block_position);        // the lowest key its first token sees
+    const int block_last_low = low_of(max(block_last, 0));       // and its last token
     const int index = min(column, max(block_valid - 1, 0));                // columns past the end repeat the last token
     const int my_position = block_position + index;
-    const int my_low = window > 0 ? max(0, my_position - window + 1) : 0;
+    const int my_low = low_of(my_position);
 
     PFrag8 q_frag[K_STEPS];
 #pragma unroll
@@ -480,7 +485,9 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
 
     // o_acc[d][i]: dim 32 d + 8 (i / 4) + 4 half + i % 4 of token `column`.
     if (column < block_valid) {
-        const float inverse = (EXTRA ? extras.out_scale : 1.0f) / running_sum;
+        float inverse = (EXTRA ? extras.out_scale : 1.0f) / running_sum;
+        if (EXTRA && extras.gate != nullptr)        // the head's gate: sigmoid of one number a token and head
+            inverse *= 1.0f / (1.0f + __expf(-extras.gate[static_cast<int64_t>(first_token + block_first + column) * extras.gate_stride + head]));
         bf16* out_row = EXTRA ? out + static_cast<int64_t>(first_token + block_first + column) * extras.out_stride + head * HD
                               : out + (static_cast<int64_t>(first_token + block_first + column) * heads + head) * HD;
 #pragma unroll

@@ -244,6 +244,9 @@ typedef struct MllAttentionExtras {
     const float* sink;
     float out_scale;
     int64_t out_stride;
+    int chunk;              // > 0 (and no window): a query at p sees the keys from floor(p / chunk) * chunk on
+    const float* gate;      // null, or float32 rows gate_stride apart, one number a head: the head's result times sigmoid(gate[t][head])
+    int64_t gate_stride;
 } MllAttentionExtras;
 
 int mll_paged_attention_decode_extra(const void* q, const void* k_cache, const void* v_cache,

@@ -682,16 +682,21 @@ def gemm_bf16_split(x: torch.Tensor, weight: torch.Tensor, parts: int) -> torch.
 
 class _AttentionExtras(ctypes.Structure):
     _fields_ = [("bias", ctypes.c_void_p), ("longest", ctypes.c_int), ("sink", ctypes.c_void_p),
-                ("out_scale", ctypes.c_float), ("out_stride", ctypes.c_int64)]
+                ("out_scale", ctypes.c_float), ("out_stride", ctypes.c_int64), ("chunk", ctypes.c_int), ("gate", ctypes.c_void_p),
+                ("gate_stride", ctypes.c_int64)]
 
 
 class AttentionExtras(NamedTuple):
     """What the MFMA attention kernels take beyond scale and window: ``bias`` float32 ``[distances, heads]`` added to
     the scaled scores by ``min(distance, last row)``; ``sink`` float32 ``[heads]``, one more term ``exp(sink)`` of the
-    softmax's denominator; a factor on the result."""
+    softmax's denominator; a factor on the result; ``chunk``: a query at ``p`` sees the keys from ``floor(p / chunk) *
+    chunk`` on (no window then); ``gate`` float32 ``[tokens, heads]`` (columns of a wider buffer allowed): a head's result
+    is multiplied by ``sigmoid(gate)``."""
     bias: Optional[torch.Tensor] = None
     sink: Optional[torch.Tensor] = None
     out_scale: float = 1.0
+    chunk: int = 0
+    gate: Optional[torch.Tensor] = None
 
 
 def prefill_bias_rows() -> int:
@@ -713,9 +718,17 @@ def _extras_argument(extras: Optional[AttentionExtras], heads: int, head_dim: in
         _need(tuple(extras.sink.shape) == (heads,), "one sink a head")
     _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == heads * head_dim, "the output is [tokens, heads * head_dim] with unit column stride")
     stride = max(out.stride(0), heads * head_dim)
+    gate_stride = 0
+    if extras.gate is not None:
+        gate = extras.gate
+        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and tuple(gate.shape) == (out.shape[0], heads)
+              and gate.stride(1) == 1, "the gate is float32 [tokens, heads] with unit column stride")
+        gate_stride = max(gate.stride(0), heads)
+    _need(extras.chunk >= 0, "chunks of positions are positive, or 0 for none")
     return ctypes.byref(_AttentionExtras(extras.bias.data_ptr() if extras.bias is not None else None, longest,
                                          extras.sink.data_ptr() if extras.sink is not None else None,
-                                         float(extras.out_scale), stride))
+                                         float(extras.out_scale), stride, int(extras.chunk),
+                                         extras.gate.data_ptr() if extras.gate is not None else None, gate_stride))
 
 
 def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
@@ -834,9 +847,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     """
     mfma_fits = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
     _need(mfma_fits or (extras is None and out is None), "a bias, a sink or an output of its own need the MFMA kernels")
+    _need(extras is None or not (extras.chunk and window), "a window or chunks of positions, not both")
     if mfma_fits and ctx.max_count == 1:
         longest = max(ctx.planned_total, ctx.max_total)
-        visible = min(longest, window) if window > 0 else longest
+        reach = window if window > 0 else (extras.chunk if extras is not None else 0)      # the most keys a query sees, 0: all
+        visible = min(longest, reach) if reach > 0 else longest
         splits = decode_splits(ctx.n_tokens, kv_heads, visible)
         return paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                       scale, window, heads, kv_heads, head_dim, splits, out=out, extras=extras)
@@ -851,7 +866,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                     scale, window, heads, kv_heads, head_dim, out=out, extras=extras)
         if plan.single_tokens.shape[0] > 0:
             longest = max(plan.max_single_total, ctx.planned_total) if ctx.fixed else plan.max_single_total
-            visible = min(longest, window) if window > 0 else longest
+            reach = window if window > 0 else (extras.chunk if extras is not None else 0)
+            visible = min(longest, reach) if reach > 0 else longest
             splits = decode_splits(plan.single_tokens.shape[0], kv_heads, visible)
             paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=plan.single_tokens,
@@ -1120,7 +1136,7 @@ def embedding_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.
     _need(tuple(rates.shape) == ((width + 1) // 2,), "one rate per pair of columns")
     out = torch.empty((ids.shape[0], width), dtype=torch.float32, device=table.device)
     _check(lib.mll_embedding_sinusoid(_ptr(table), _code(table.dtype), _ptr(ids), _ptr(positions), _ptr(rates), _ptr(out),
-                                      ids.shape[0], width, vocab, ctypes.c_float(scale), _stream()), lib)
+                                      ids.shape[0], width, vocab, _stream()), lib)
     return out
 
 

@@ -105,9 +105,8 @@ class BucketBiasAttention(Mixer):
         if self.slope_values is None and not self.bias_rows:
             table_rows = 1      # no table at all
         self.tiled = (bool(p.get("mfma", True)) and runtime.dtype == torch.bfloat16 and self.key_dim == self.value_dim
-                      and self.key_dim % 16 == 0 and self.key_dim <= 256 and 0 < table_rows <= kernels.MFMA_BIAS_ROWS
-                      and not self.chunk and not self.head_gate)
-        self.planner = QueryTilePlanner(bool(self.window)) if self.tiled else None
+                      and self.key_dim % 16 == 0 and self.key_dim <= 256 and 0 < table_rows <= kernels.MFMA_BIAS_ROWS)
+        self.planner = QueryTilePlanner(bool(self.window or self.chunk)) if self.tiled else None
         self.slopes = self.o_bias = self.qkv_bias = None
         self.qkv_weight: Optional[Weight] = None
         self.o_tensor: Optional[torch.Tensor] = None
@@ -218,7 +217,7 @@ class BucketBiasAttention(Mixer):
         if self.tiled:
             if out is None:
                 out = torch.empty((x.shape[0], self.heads * self.value_dim), dtype=self.runtime.dtype, device=x.device)
-            extras = kernels.AttentionExtras(self.bias, self.sink, out_scale)
+            extras = kernels.AttentionExtras(self.bias, self.sink, out_scale, chunk=self.chunk, gate=gate)
             return kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, self.window, self.heads, self.kv_heads,
                                            self.key_dim, planner=self.planner, extras=extras, out=out)
         return kernels.bias_attention(q, cache.k, cache.v, view.block_table, ctx.seq_of_token, ctx.positions, self.bias,

@@ -48,6 +48,8 @@ class RoutedExperts(FeedForward):
         self.keep_groups = int(p.get("keep_groups") or 0)
         if p.get("expert_form", "gated") not in ("gated", "plain") or self.activation not in kernels.ACTIVATIONS:
             raise ValueError("expert_form is gated or plain, activation one of " + ", ".join(kernels.ACTIVATIONS))
+        if self.gated and self.shared_size and self.activation != "silu":
+            raise ValueError("a gated shared expert takes SiLU: the products' gated epilogue has no other activation")
         if self.groups and (self.experts % self.groups or not 1 <= self.keep_groups <= self.groups
                             or self.keep_groups * (self.experts // self.groups) < self.top):
             raise ValueError("equal groups of experts, of which the kept ones hold at least `top` experts")
@@ -129,10 +131,8 @@ class RoutedExperts(FeedForward):
         kernels.moe_experts(x, ids, weights, self.gate_up, self.down, self.weight_on == "input", out=parts, gated=self.gated,
                             activation=self.activation)
         if self.shared_size:
-            if self.gated and self.activation == "silu":
+            if self.gated:
                 inner = linear(x, self.shared_gate_up, gated=True)
-            elif self.gated:
-                raise NotImplementedError("a gated shared expert with an activation other than SiLU")
             else:       # the activation reads the product's float32 sums and rounds once
                 inner = kernels.activation(linear(x, self.shared_gate_up, out_dtype=torch.float32, partials=True), self.activation, x.dtype)
             if shared_factor is not None:

@@ -8,7 +8,9 @@ the keys ``j`` with ``0 <= p - j < window``, scores are ``(q_flat . Wuk_h c_j + 
 is the ordinary one, the heads side by side are multiplied by ``sigmoid(Wg x)`` (``output_gate``) and projected by
 ``Wo``. A layer with ``owns_kv`` False has no ``Wdkv``: it reads the latents another run entry cached. Without a
 ``q_rank`` the queries have no latent: ``q = Wq x``. With ``gate_a_head`` the gate is one number a head, ``Wg`` being
-``[heads, hidden]``.
+``[heads, hidden]``. With a position encoding that turns neighbouring channels together (``rope_neighbours``) the rows
+of ``Wq`` (or ``Wuq``) and ``Wdkv`` that make the turned parts are brought into split-half order once, at load: the turned
+parts of queries and keys only ever meet in their dot product, which does not change when both are reordered alike.
 
 Only ``[c | kr]`` is cached, one row a token. The up projections are folded into the query and into the result:
 ``q'_h = Wuk_h^T q_flat`` (``kv_rank`` numbers) and ``o_h = Wuv_h sum_j p_j c_j``, so the attention has a single kv

@@ -99,31 +99,48 @@ def latent_attention(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps:
     return out.reshape(T, H * vdim) @ t64(tensors, f"{prefix}.o").T
 
 
-def chunked_sink_attention(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps: float) -> torch.Tensor:
-    T = a.shape[0]
-    H, G, dim, vdim = mixer["heads"], mixer["kv_heads"], mixer["dim"], mixer["vdim"]
-    size = mixer["mask"]["size"]
-    rot = mixer["rot"]
-    divide = rot.get("scaling", {}).get("factor", 1.0) if rot.get("scaling") else 1.0
-    positions = torch.arange(T)
-    q = (a @ t64(tensors, f"{prefix}.q").T).view(T, H, dim)
-    k = (a @ t64(tensors, f"{prefix}.k").T).view(T, G, dim)
-    v = (a @ t64(tensors, f"{prefix}.v").T).view(T, G, vdim)
-    q = rms(q, eps) * t64(tensors, f"{prefix}.q.norm")
-    k = rms(k, eps) * t64(tensors, f"{prefix}.k.norm")
-    q = turn_halves(q, positions, rot["base"], rot["dims"], divide)
-    k = turn_halves(k, positions, rot["base"], rot["dims"], divide)
-    gate = torch.sigmoid(a @ t64(tensors, f"{prefix}.g").T)          # [T, H]
-    out = torch.zeros(T, H, vdim, dtype=F)
+def attend_in_chunks(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, size: int) -> torch.Tensor:
+    """``q`` ``[T, H, d]``, ``k`` ``[T, G, d]``, ``v`` ``[T, G, dv]`` as they enter the scores. Position ``i`` sees ``j <= i``
+    of its own chunk of ``size`` positions; the weights are ``exp(s_j) / (1 + sum exp(s))``."""
+    T, H = q.shape[0], q.shape[1]
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=F)
     for i in range(T):
         first = (i // size) * size
         for h in range(H):
             g = h // (H // G)
-            s = (k[first: i + 1, g] @ q[i, h]) * mixer["scale"]
+            s = (k[first: i + 1, g] @ q[i, h]) * scale
             w = torch.exp(s)
-            p = w / (1.0 + w.sum())
-            out[i, h] = (p[:, None] * v[first: i + 1, g]).sum(0) * gate[i, h]
+            out[i, h] = ((w / (1.0 + w.sum()))[:, None] * v[first: i + 1, g]).sum(0)
+    return out
+
+
+def chunked_sink_attention(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps: float) -> torch.Tensor:
+    T = a.shape[0]
+    H, G, dim, vdim = mixer["heads"], mixer["kv_heads"], mixer["dim"], mixer["vdim"]
+    rot = mixer["rot"]
+    divide = rot["scaling"]["factor"] if rot.get("scaling") else 1.0
+    positions = torch.arange(T)
+    q = (a @ t64(tensors, f"{prefix}.q").T).view(T, H, dim)
+    k = (a @ t64(tensors, f"{prefix}.k").T).view(T, G, dim)
+    v = (a @ t64(tensors, f"{prefix}.v").T).view(T, G, vdim)
+    q = turn_halves(rms(q, eps) * t64(tensors, f"{prefix}.q.norm"), positions, rot["base"], rot["dims"], divide)
+    k = turn_halves(rms(k, eps) * t64(tensors, f"{prefix}.k.norm"), positions, rot["base"], rot["dims"], divide)
+    out = attend_in_chunks(q, k, v, mixer["scale"], mixer["mask"]["size"])
+    out = out * torch.sigmoid(a @ t64(tensors, f"{prefix}.g").T)[:, :, None]       # one gate a head
     return out.reshape(T, H * vdim) @ t64(tensors, f"{prefix}.o").T
+
+
+def retain(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay, state: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``S <- decay_h S + k v^T``, ``o = S^T q`` token by token; ``q``, ``k`` ``[T, H, d]``, ``v`` ``[T, H, dv]``."""
+    T, H, dim = q.shape
+    decay = torch.as_tensor(decay, dtype=F)
+    state = torch.zeros(H, dim, v.shape[2], dtype=F) if state is None else state.clone()
+    out = torch.zeros(T, H, v.shape[2], dtype=F)
+    for t in range(T):
+        state = decay[:, None, None] * state + k[t][:, :, None] * v[t][:, None, :]
+        out[t] = torch.einsum("hdv,hd->hv", state, q[t])
+    return out
 
 
 def retention(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps: float) -> torch.Tensor:
@@ -132,13 +149,7 @@ def retention(a: torch.Tensor, tensors, prefix: str, mixer: Mapping, eps: float)
     q = (a @ t64(tensors, f"{prefix}.q").T).view(T, H, dim)
     k = (a @ t64(tensors, f"{prefix}.k").T).view(T, H, dim) * dim ** -0.5
     v = (a @ t64(tensors, f"{prefix}.v").T).view(T, H, vdim)
-    decay = torch.tensor(mixer["decay"], dtype=F)
-    state = torch.zeros(H, dim, vdim, dtype=F)
-    out = torch.zeros(T, H, vdim, dtype=F)
-    for t in range(T):
-        state = decay[:, None, None] * state + k[t][:, :, None] * v[t][:, None, :]
-        out[t] = torch.einsum("hdv,hd->hv", state, q[t])
-    out = rms(out, eps).reshape(T, H * vdim) * silu(a @ t64(tensors, f"{prefix}.g").T)
+    out = rms(retain(q, k, v, mixer["decay"]), eps).reshape(T, H * vdim) * silu(a @ t64(tensors, f"{prefix}.g").T)
     return out @ t64(tensors, f"{prefix}.o").T
 
 
@@ -219,7 +230,7 @@ def forward(config: Mapping, tensors: Mapping[str, torch.Tensor], ids, layers_ou
     """Logits ``[T, vocab]`` (float64) of one sequence run whole."""
     eps = config["norm"]["eps"]
     ids = torch.as_tensor(ids, dtype=torch.int64)
-    e = t64(tensors, "embed")[ids] * config["embedding"]["scale"]
+    e = t64(tensors, "embed")[ids] * (config.get("embedding") or {}).get("scale", 1.0)
     x = e.clone()
     for index, again in run_order(config):
         layer = config["layers"][index]
@@ -248,3 +259,25 @@ def forward(config: Mapping, tensors: Mapping[str, torch.Tensor], ids, layers_ou
             layers_out.append(x.clone())
     x = rms(x, eps) * t64(tensors, "final.norm")
     return x @ t64(tensors, "head").T
+
+
+def read_config(folder: str) -> dict:
+    import json
+    import os
+    with open(os.path.join(folder, "config.json"), "r", encoding="utf-8") as handle:
+        return json.load(handle)
+
+
+def read_tensors(folder: str) -> Dict[str, torch.Tensor]:
+    import os
+    from safetensors.torch import load_file
+    return load_file(os.path.join(folder, "model.safetensors"))
+
+
+def generate_greedy(config: Mapping, tensors: Mapping[str, torch.Tensor], prompt: List[int], count: int) -> List[int]:
+    """``count`` tokens after ``prompt``, each the first maximum of the last position's logits; every step runs the
+    whole sequence again."""
+    tokens = list(prompt)
+    for _ in range(count):
+        tokens.append(int(torch.argmax(forward(config, tensors, tokens)[-1])))
+    return tokens[len(prompt):]
