@@ -16,7 +16,7 @@ namespace mll {
 
 constexpr int kMaxTop = 16;
 
-// One thread a token. z: float32 rows, z_stride apart, experts first; a further column `shared_at` (negative: none)
+// One thread a token (taken beyond 256 experts; fewer go to the kernel below, a wave a token). z: float32 rows, z_stride apart, experts first; a further column `shared_at` (negative: none)
 // holds the logit of the shared expert's gate, whose sigmoid goes to shared_gate[t].
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const float* __restrict__ z, int64_t z_stride, int n_tokens, int experts, int top, int softmax_scores,
@@ -77,6 +77,106 @@ moe_route_kernel(const float* __restrict__ z, int64_t z_stride, int n_tokens, in
         weights[static_cast<int64_t>(token) * top + n] = renormalize ? taken[n] / sum : taken[n];
     }
     if (shared_at >= 0 && shared_gate != nullptr) shared_gate[token] = 1.0f / (1.0f + expf(-row[shared_at]));
+}
+
+// The same choice by one wave a token, for up to 64 * PER experts: lane l holds the experts l, l + 64, ...; maxima,
+// sums and every "largest of what is left" are taken across the wave, ties to the lower index. The scores' sum is
+// added in the wave's order, not in the experts'; everything else is the arithmetic of the kernel above, and a token's
+// result depends on its own row alone.
+struct Candidate {
+    float value;
+    int index;
+};
+
+__device__ inline Candidate wave_best(Candidate mine) {
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+        const float value = __shfl_xor(mine.value, offset, kWave);
+        const int index = __shfl_xor(mine.index, offset, kWave);
+        const bool better = index >= 0 && (mine.index < 0 || value > mine.value || (value == mine.value && index < mine.index));
+        if (better) {
+            mine.value = value;
+            mine.index = index;
+        }
+    }
+    return mine;
+}
+
+template <int PER>
+__global__ void __launch_bounds__(kWave)
+moe_route_wave_kernel(const float* __restrict__ z, int64_t z_stride, int experts, int top, int softmax_scores, int renormalize,
+                      int shared_at, int32_t* __restrict__ ids, float* __restrict__ weights, float* __restrict__ shared_gate,
+                      int groups, int keep) {
+    const int token = blockIdx.x, lane = threadIdx.x;
+    const float* row = z + static_cast<int64_t>(token) * z_stride;
+    float logit[PER];
+    bool free_to_take[PER];
+    float peak = -INFINITY;
+#pragma unroll
+    for (int n = 0; n < PER; ++n) {
+        const int e = lane + n * kWave;
+        const float value = e < experts ? row[e] : -INFINITY;
+        logit[n] = value != value ? -INFINITY : value;       // a logit that is no number is never the largest
+        free_to_take[n] = e < experts;
+        peak = fmaxf(peak, logit[n]);
+    }
+    float total = 1.0f;
+    if (softmax_scores) {
+        peak = wave_max(peak);
+        float part = 0.0f;
+#pragma unroll
+        for (int n = 0; n < PER; ++n)
+            if (lane + n * kWave < experts) part += expf(logit[n] - peak);
+        total = wave_sum(part);
+    }
+    if (groups > 0 && keep < groups) {
+        // lane g learns group g's largest logit; then the best `keep` groups are opened, one after the other
+        const int group_size = experts / groups;
+        float group_top = -INFINITY;
+        for (int g = 0; g < groups; ++g) {
+            float inside = -INFINITY;
+#pragma unroll
+            for (int n = 0; n < PER; ++n) {
+                const int e = lane + n * kWave;
+                if (e < experts && e / group_size == g) inside = fmaxf(inside, logit[n]);
+            }
+            inside = wave_max(inside);
+            if (lane == g) group_top = inside;
+        }
+        unsigned long long open_groups = 0ull;
+        for (int n = 0; n < keep; ++n) {
+            Candidate mine = {group_top, (lane < groups && !((open_groups >> lane) & 1ull)) ? lane : -1};
+            open_groups |= 1ull << wave_best(mine).index;
+        }
+#pragma unroll
+        for (int n = 0; n < PER; ++n) {
+            const int e = lane + n * kWave;
+            free_to_take[n] = free_to_take[n] && ((open_groups >> (e / group_size)) & 1ull);
+        }
+    }
+    float sum = 0.0f, my_weight = 0.0f;
+    int my_id = 0;
+    for (int choice = 0; choice < top; ++choice) {
+        Candidate mine = {-INFINITY, -1};
+#pragma unroll
+        for (int n = 0; n < PER; ++n)       // ascending index: of equal logits the lower stays
+            if (free_to_take[n] && (mine.index < 0 || logit[n] > mine.value)) mine = {logit[n], lane + n * kWave};
+        const Candidate best = wave_best(mine);
+#pragma unroll
+        for (int n = 0; n < PER; ++n)
+            if (lane + n * kWave == best.index) free_to_take[n] = false;
+        const float taken = softmax_scores ? expf(best.value - peak) / total : 1.0f / (1.0f + expf(-best.value));
+        sum += taken;
+        if (lane == choice) {
+            my_weight = taken;
+            my_id = best.index;
+        }
+    }
+    if (lane < top) {
+        ids[static_cast<int64_t>(token) * top + lane] = my_id;
+        weights[static_cast<int64_t>(token) * top + lane] = renormalize ? my_weight / sum : my_weight;
+    }
+    if (lane == 0 && shared_at >= 0 && shared_gate != nullptr) shared_gate[token] = 1.0f / (1.0f + expf(-row[shared_at]));
 }
 
 template <typename T> __device__ inline float row_dot(const T* __restrict__ w, const float* __restrict__ x, int k, int lane);
@@ -475,8 +575,16 @@ int mll_moe_route(const float* z, int64_t z_stride, int n_tokens, int experts, i
                                 keep * (experts / groups) >= top),
                 "moe_route: at most 64 equal groups, of which the kept ones hold at least `top` experts");
     if (n_tokens == 0) return 0;
-    moe_route_kernel<<<(n_tokens + 63) / 64, 64, 0, stream>>>(z, z_stride, n_tokens, experts, top, softmax_scores, renormalize,
-                                                            shared_at, ids, weights, shared_gate, groups, keep);
+#define MLL_ROUTE_WAVE(PER)                                                                                                  \
+    moe_route_wave_kernel<PER><<<n_tokens, kWave, 0, stream>>>(z, z_stride, experts, top, softmax_scores, renormalize, shared_at, \
+                                                              ids, weights, shared_gate, groups, keep)
+    if (experts <= kWave) MLL_ROUTE_WAVE(1);
+    else if (experts <= 2 * kWave) MLL_ROUTE_WAVE(2);
+    else if (experts <= 4 * kWave) MLL_ROUTE_WAVE(4);
+    else
+        moe_route_kernel<<<(n_tokens + 63) / 64, 64, 0, stream>>>(z, z_stride, n_tokens, experts, top, softmax_scores, renormalize,
+                                                                shared_at, ids, weights, shared_gate, groups, keep);
+#undef MLL_ROUTE_WAVE
     return check_launch("moe_route");
 }
 

@@ -371,7 +371,7 @@ def test_a_far_token_stays_in_the_state():
         assert np.abs(got[n - 1, 1]).max() < 1e-20 / 1e-5 ** 0.5, portions_of
 
 
-@pytest.mark.parametrize("experts,top,groups,keep", [(8, 2, 4, 2), (12, 4, 4, 3), (6, 1, 3, 1), (16, 4, 4, 4), (5, 3, 0, 0), (12, 3, 6, 2), (64, 6, 8, 3)])
+@pytest.mark.parametrize("experts,top,groups,keep", [(8, 2, 4, 2), (12, 4, 4, 3), (6, 1, 3, 1), (16, 4, 4, 4), (5, 3, 0, 0), (12, 3, 6, 2), (64, 6, 8, 3), (100, 6, 10, 4), (300, 8, 0, 0)])
 def test_choice_of_experts_among_the_best_groups(experts, top, groups, keep):
     from microllm_rocm_amd.ops import kernels
     rng = np.random.default_rng(experts + top)
