@@ -569,7 +569,8 @@ extern "C" {
 int mll_moe_route(const float* z, int64_t z_stride, int n_tokens, int experts, int top, int softmax_scores, int renormalize,
                   int shared_at, int32_t* ids, float* weights, float* shared_gate, int groups, int keep, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && experts > 0 && top > 0 && top <= experts, "moe_route: 1 <= top <= experts");
-    MLL_REQUIRE(top <= kMaxTop, "moe_route: more than 16 experts a token are not supported");
+    MLL_REQUIRE(top <= (experts <= 4 * kWave ? kWave : kMaxTop),
+                "moe_route: at most 64 experts a token (16 where there are more than 256 experts)");
     MLL_REQUIRE(shared_at < 0 || shared_gate != nullptr, "moe_route: the shared expert's gate needs a place");
     MLL_REQUIRE(groups == 0 || (groups > 0 && groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups &&
                                 keep * (experts / groups) >= top),
