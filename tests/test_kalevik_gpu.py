@@ -148,6 +148,33 @@ def test_rows_that_join_the_stream_with_a_normed_delta(width):
     assert np.abs(got.cpu().numpy() - want[[4, 1]]).max() < 2e-5
 
 
+def test_rows_join_the_stream_whatever_the_layer_before_left():
+    """``Model`` adds the embedding's rows before an entry that asks for them: along with a delta that is still to be
+    normed, or at once where the delta is plain (another arrangement) or there is none."""
+    from microllm_rocm_amd.parts.model import Model
+    from microllm_rocm_amd.parts.norm import NormedDelta
+    rng = np.random.default_rng(9)
+    h, delta, rows = (rng.normal(size=(5, 24)) for _ in range(3))
+    stream = device(h)
+    assert Model._add_to_stream(stream, None, device(rows)) is None
+    assert np.abs(stream.cpu().numpy() - (h + rows)).max() < 1e-6
+    stream = device(h)
+    assert Model._add_to_stream(stream, device(delta), device(rows)) is None
+    assert np.abs(stream.cpu().numpy() - (h + delta + rows)).max() < 1e-6
+    stream, parts = device(h), device(np.stack([delta * 0.25, delta * 0.75]))
+    assert Model._add_to_stream(stream, parts, device(rows)) is None
+    assert np.abs(stream.cpu().numpy() - (h + delta + rows)).max() < 1e-6
+    stream = device(h)
+    normed = NormedDelta(device(delta), device(np.ones(24)), 1e-5, 1.0)
+    taken = Model._add_to_stream(stream, normed, device(rows))
+    assert isinstance(taken, NormedDelta) and taken.extra is not None and normed.extra is None
+    assert np.array_equal(stream.cpu().numpy(), device(h).cpu().numpy())       # nothing added yet: the next norm's kernel does it
+    want = t64(rows) + plain.rms(t64(delta), 1e-5)
+    assert np.abs(taken.resolved().cpu().numpy() - want.numpy()).max() < 1e-5
+    with pytest.raises(ValueError):
+        taken.with_extra(device(rows))
+
+
 def test_activations_by_name():
     from microllm_rocm_amd.ops import kernels
     z = np.random.default_rng(2).normal(size=(5, 33)) * 3
