@@ -130,12 +130,12 @@ def kalevik_config(size: dict):
     width, heads, kv_heads, dim, ff = size["width"], size["heads"], size["kv_heads"], size["head_dim"], size["ff"]
     latent = LatentAttentionConfig(heads=heads, dim=96, rot_dim=64, vdim=dim, kv_rank=192, scale=160 ** -0.5, rot_base=1e6, rot_dims=64)
     left = ChunkAttentionConfig(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, chunk=8192, rot_base=1e6,
-                                rot_dims=dim // 2, rot_factor=4.0)
-    right = RetentionConfig(heads=heads // 2, dim=dim // 2, vdim=dim, decay=tuple(1.0 - 2.0 ** (-5 - head % 6) for head in range(heads // 2)))
+                                rot_dims=dim // 2, rot_factor=2.0)
+    right = RetentionConfig(heads=heads // 2, dim=dim // 2, vdim=dim, decay=tuple(1.0 - 0.1 / (1 + head % 6) for head in range(heads // 2)))
     moe = MoeMlpConfig(experts=16, top=4, expert_ff=ff // 4, groups=4, keep_groups=2, shared_ff=ff // 2)
     layers = [KalevikLayerConfig("latent_attention", latent, DenseMlpConfig(ff)) if index % 2 == 0 else
-              KalevikLayerConfig("parallel", ParallelConfig(left, right, 0.6, 0.9), moe) for index in range(size["layers"])]
-    return KalevikConfig(vocab=DESIGN_VOCAB, width=width, norm_eps=1e-6, layers=tuple(layers), embedding_scale=3.0)
+              KalevikLayerConfig("parallel", ParallelConfig(left, right, 0.75, 1.25), moe) for index in range(size["layers"])]
+    return KalevikConfig(vocab=DESIGN_VOCAB, width=width, norm_eps=1e-6, layers=tuple(layers), embedding_scale=2.0)
 
 
 def design_configs(size: dict, design: str = "siditar"):

@@ -62,7 +62,7 @@ TINY_B = KalevikConfig(
 TINY_C = KalevikConfig(
     vocab=150, width=96, norm_eps=1e-6, embedding_scale=0.5, loop=LoopConfig(0, 2, 3),
     layers=(
-        _layer(ParallelConfig(_left(8, 2, 32, 32, 0.18, 17, 16, factor=4.0), _right(16, 24, [0.5, 0.75, 0.875]), 0.6, 0.9),
+        _layer(ParallelConfig(_left(8, 2, 32, 32, 0.18, 17, 16, factor=3.0), _right(16, 24, [0.5, 0.75, 0.875]), 0.75, 1.25),
                MoeMlpConfig(experts=16, top=4, expert_ff=64, groups=4, keep_groups=4, shared_ff=32)),
         _layer(_latent(5, 24, 32, 40, 224, 0.15, base=500.0), 128),
         _layer(ParallelConfig(_left(2, 1, 24, 40, 0.3, 1, 24), _right(128, 12, [0.96]), 1.0, 0.8),
