@@ -65,7 +65,6 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
         const int i = ROWS * r + m;
         s[m] = i < key_dim ? mine[static_cast<int64_t>(i) * value_dim] : 0.0f;
     }
-    const int channels = heads * key_dim;
     float a_next[ROWS], k_next[ROWS], q_next[ROWS], v_next;
     auto fetch = [&](int token) {
         const float* row = proj + static_cast<int64_t>(token) * proj_stride;
@@ -166,7 +165,6 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
 #pragma unroll
     for (int m = 0; m < ROWS; ++m) all_valid = all_valid && valid[m];
     all_valid = __all(all_valid);
-    const int channels = heads * key_dim;
     const int value_calls = (tile_tokens * columns + kWave - 1) / kWave;
     auto fetch = [&](int tile_first, float* buffer) __attribute__((always_inline)) {
 #pragma unroll

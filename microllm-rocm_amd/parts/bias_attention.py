@@ -102,8 +102,6 @@ class BucketBiasAttention(Mixer):
         # slopes are such a column only under a window that fits)
         # (the widest window among the layers that share the pages decides, so that all of them lay the pages out alike)
         table_rows = self.kept_window if self.slope_values is not None else self.bias_max + 1
-        if self.slope_values is None and not self.bias_rows:
-            table_rows = 1      # no table at all
         self.tiled = (bool(p.get("mfma", True)) and runtime.dtype == torch.bfloat16 and self.key_dim == self.value_dim
                       and self.key_dim % 16 == 0 and self.key_dim <= 256 and 0 < table_rows <= kernels.MFMA_BIAS_ROWS)
         self.planner = QueryTilePlanner(bool(self.window or self.chunk)) if self.tiled else None
